@@ -1,0 +1,76 @@
+"""Small seeded graphs shared by the CPU and GPU tests, with the edge cases the
+reference's API allows: empty rows, duplicate edges, a hub row, rectangular
+matrices, m < rows, and pntrb/pntre that are not rowptr / rowptr+1."""
+import numpy as np
+
+from fusedmm_amd import synth
+
+
+def tiny_er(n=200, pairs=800, seed=11, bits=32):
+    return synth.er_graph(n, pairs, seed, bits)
+
+
+def with_values(g, seed=7):
+    g = dict(g)
+    g["val"] = synth.edge_values(g["nnz"], seed)
+    return g
+
+
+def ragged(bits=32, seed=3, rows=97, cols=131, hub_deg=600):
+    """Rectangular, rows 0 and 5 and the last one empty, a duplicate column in
+    row 2, one hub row much longer than the rest (with repeats), unsorted row 7."""
+    rng = np.random.Generator(np.random.Philox(key=[seed, 0]))
+    it = np.int32 if bits == 32 else np.int64
+    lists = []
+    for r in range(rows):
+        if r in (0, 5, rows - 1):
+            lists.append(np.empty(0, np.int64))
+        elif r == 2:
+            lists.append(np.array([4, 9, 9, 30], np.int64))
+        elif r == 7:
+            lists.append(np.array([50, 3, 77, 12, 3], np.int64))
+        elif r == 11:
+            lists.append(rng.integers(0, cols, hub_deg, dtype=np.int64))
+        else:
+            d = int(rng.integers(1, 24))
+            lists.append(np.sort(rng.choice(cols, d, replace=False)).astype(np.int64))
+    deg = np.array([len(x) for x in lists], np.int64)
+    rowptr = np.zeros(rows + 1, np.int64)
+    np.cumsum(deg, out=rowptr[1:])
+    indx = np.concatenate(lists)
+    g = synth.graph_from_rowptr(rows, cols, rowptr, indx, None, bits)
+    g["val"] = synth.edge_values(g["nnz"], seed)
+    assert g["indx"].dtype == it
+    return g
+
+
+def split_pointers(g, seed=5):
+    """Same rows, but stored with gaps and in shuffled order: pntrb[i]/pntre[i]
+    point into a longer indx/val with junk between rows (pntre[i] != pntrb[i+1])."""
+    rng = np.random.Generator(np.random.Philox(key=[seed, 1]))
+    rows = g["rows"]
+    deg = (g["pntre"] - g["pntrb"]).astype(np.int64)
+    order = rng.permutation(rows)
+    gap = rng.integers(0, 4, rows)
+    total = int(deg.sum() + gap.sum()) + 3
+    indx = np.full(total, 0, g["indx"].dtype)       # junk points at a valid row of Y
+    val = np.full(total, np.float32(1e30))          # ... but would wreck Z if read
+    pb = np.zeros(rows, g["indx"].dtype)
+    pe = np.zeros(rows, g["indx"].dtype)
+    pos = 3
+    for r in order:
+        pos += int(gap[r])
+        pb[r] = pos
+        d = int(deg[r])
+        indx[pos:pos + d] = g["indx"][g["pntrb"][r]:g["pntre"][r]]
+        val[pos:pos + d] = g["val"][g["pntrb"][r]:g["pntre"][r]]
+        pos += d
+        pe[r] = pos
+    out = dict(g)
+    out.update(indx=indx, val=val, pntrb=pb, pntre=pe, nnz=total)
+    out.pop("rowptr", None)
+    return out
+
+
+def features(n, k, seed, lo=-0.5, hi=0.5, stream=1):
+    return synth.uniform_matrix(n, k, lo, hi, seed, stream)
