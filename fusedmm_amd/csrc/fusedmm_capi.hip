@@ -1,0 +1,657 @@
+// C-ABI layer of libfusedmm_amd_i{32,64}.so: decodes the op tuple, picks the
+// kernel instance for (K, alignment, op), keeps the per-device work queues and
+// staging buffers, and launches the gfx950 kernels of fusedmm_kernels.h.
+//
+// Replaces the dispatch of the reference's fusedMM.c:487-744 and
+// kernels/src/kernels.c:456-631.  Built once per index width (-DINDEXTYPE=...).
+#include <hip/hip_runtime.h>
+#include <dlfcn.h>
+#include <math.h>
+#include <stdint.h>
+#include <stdio.h>
+#include <stdlib.h>
+#include <string.h>
+
+#include <mutex>
+#include <vector>
+
+#ifndef INDEXTYPE
+#error "compile with -DINDEXTYPE=int32_t or -DINDEXTYPE=int64_t"
+#endif
+#define VALUETYPE float
+#include "../../include/fusedMM.h"
+#include "../../include/fusedmm_amd.h"
+#include "fusedmm_kernels.h"
+
+namespace {
+
+using namespace fmm;
+typedef INDEXTYPE idx_t;
+
+#define FMM_LOG(...)                                   \
+   do {                                                \
+      fprintf(stderr, "fusedmm_amd: " __VA_ARGS__);    \
+      fprintf(stderr, "\n");                           \
+   } while (0)
+
+// hipError -> reference status code (fusedMM.h:103-112)
+inline int hip_status(hipError_t e, const char *what)
+{
+   if (e == hipSuccess) return FUSEDMM_SUCCESS_RETURN;
+   FMM_LOG("%s failed: %s", what, hipGetErrorString(e));
+   (void)hipGetLastError();
+   return e == hipErrorOutOfMemory ? FUSEDMM_NOT_ENOUGH_MEM : FUSEDMM_FAIL_RETURN;
+}
+#define FMM_HIP(call)                                  \
+   do {                                                \
+      int st_ = hip_status((call), #call);             \
+      if (st_ != FUSEDMM_SUCCESS_RETURN) return st_;   \
+   } while (0)
+
+constexpr int kMaxDevices = 16;
+constexpr int kTimingSlots = 512;
+constexpr int kMaxK = 2048;
+
+struct Buffer {
+   void *ptr = nullptr;
+   size_t bytes = 0;
+};
+
+struct DeviceState {
+   bool ready = false;
+   int num_cu = 0;
+   float *sigmoid_table = nullptr;
+   Counters *ctr = nullptr;
+   Buffer heavy, segs, partial;
+   Buffer stage[8];           // host-pointer mode: pntrb, pntre, indx, val, x, y, z, spare
+   // timing
+   hipEvent_t ev[kTimingSlots][4];
+   bool ev_made = false;
+};
+
+struct Globals {
+   std::mutex mu;
+   int sop_kind = FUSEDMM_SOP_KIND_HOST;
+   bool sop_kind_from_env_done = false;
+   int opt = 1;
+   int64_t heavy_deg = 0;
+   int seg_len = 0;
+   int blocks_per_cu = 0;
+   fusedMM_amd_sop_fn sop_fn = nullptr;
+   bool timing = false;
+   int timing_calls = 0;
+   int timing_dev = 0;
+   DeviceState dev[kMaxDevices];
+};
+Globals g;
+
+int sop_kind_from_name(const char *s)
+{
+   if (!s) return FUSEDMM_SOP_KIND_HOST;
+   if (!strcmp(s, "host")) return FUSEDMM_SOP_KIND_HOST;
+   if (!strcmp(s, "identity")) return FUSEDMM_SOP_KIND_IDENTITY;
+   if (!strcmp(s, "sigmoid")) return FUSEDMM_SOP_KIND_SIGMOID;
+   if (!strcmp(s, "tdist")) return FUSEDMM_SOP_KIND_TDIST;
+   if (!strcmp(s, "fr")) return FUSEDMM_SOP_KIND_FR;
+   if (!strcmp(s, "ll")) return FUSEDMM_SOP_KIND_LL;
+   if (!strcmp(s, "fa")) return FUSEDMM_SOP_KIND_FA;
+   FMM_LOG("FUSEDMM_SOP_KIND=%s is not a known kind; using host", s);
+   return FUSEDMM_SOP_KIND_HOST;
+}
+
+void read_env_once()
+{
+   if (g.sop_kind_from_env_done) return;
+   g.sop_kind_from_env_done = true;
+   if (const char *e = getenv("FUSEDMM_SOP_KIND")) g.sop_kind = sop_kind_from_name(e);
+   if (const char *e = getenv("FUSEDMM_BLOCKS_PER_CU")) g.blocks_per_cu = atoi(e);
+}
+
+// The 2048-entry sigmoid table, built with the expressions of the reference's
+// tester (test/fusedMMtime.cpp:594-604): x is a float, exp is the float
+// overload, 1 + e is a float sum, the quotient is formed in double.
+void build_sigmoid_table(float *t)
+{
+   for (int i = 0; i < kSigmoidTableSize; i++)
+   {
+      float x = (float)(2.0 * 5.0 * i / kSigmoidTableSize - 5.0);
+      float e = expf(-x);
+      float denom = 1 + e;
+      t[i] = (float)(1.0 / (double)denom);
+   }
+}
+
+int grow(Buffer &b, size_t bytes)
+{
+   if (bytes <= b.bytes) return FUSEDMM_SUCCESS_RETURN;
+   if (b.ptr) FMM_HIP(hipFree(b.ptr));
+   b.ptr = nullptr;
+   b.bytes = 0;
+   FMM_HIP(hipMalloc(&b.ptr, bytes));
+   b.bytes = bytes;
+   return FUSEDMM_SUCCESS_RETURN;
+}
+
+int device_state(DeviceState **out)
+{
+   int dev = 0;
+   FMM_HIP(hipGetDevice(&dev));
+   if (dev < 0 || dev >= kMaxDevices) return FUSEDMM_FAIL_RETURN;
+   DeviceState &d = g.dev[dev];
+   if (!d.ready)
+   {
+      hipDeviceProp_t prop;
+      FMM_HIP(hipGetDeviceProperties(&prop, dev));
+      d.num_cu = prop.multiProcessorCount > 0 ? prop.multiProcessorCount : 256;
+      float host_tab[kSigmoidTableSize];
+      build_sigmoid_table(host_tab);
+      FMM_HIP(hipMalloc((void **)&d.sigmoid_table, sizeof(host_tab)));
+      FMM_HIP(hipMemcpy(d.sigmoid_table, host_tab, sizeof(host_tab), hipMemcpyHostToDevice));
+      FMM_HIP(hipMalloc((void **)&d.ctr, sizeof(Counters)));
+      FMM_HIP(hipMemset(d.ctr, 0, sizeof(Counters)));
+      d.ready = true;
+   }
+   *out = &d;
+   return FUSEDMM_SUCCESS_RETURN;
+}
+
+// ---- kernel instance selection ---------------------------------------------------
+struct Shape {
+   int V, L, R, exact, U;
+};
+
+bool aligned16(const void *p) { return ((uintptr_t)p & 15u) == 0; }
+
+int pick_shape(int k, bool vec_ok, Shape *s)
+{
+   if (k < 1 || k > kMaxK) return FUSEDMM_FAIL_RETURN;
+   if (vec_ok)
+   {
+      if (k == 32) *s = {4, 8, 1, 1, 8};
+      else if (k == 64) *s = {4, 16, 1, 1, 8};
+      else if (k == 128) *s = {4, 32, 1, 1, 8};
+      else if (k == 256) *s = {4, 64, 1, 1, 8};
+      else if (k == 512) *s = {4, 64, 2, 1, 4};
+      else if (k <= 32) *s = {4, 8, 1, 0, 8};
+      else if (k <= 64) *s = {4, 16, 1, 0, 8};
+      else if (k <= 128) *s = {4, 32, 1, 0, 8};
+      else if (k <= 256) *s = {4, 64, 1, 0, 8};
+      else if (k <= 512) *s = {4, 64, 2, 0, 4};
+      else if (k <= 1024) *s = {4, 64, 4, 0, 2};
+      else *s = {4, 64, 8, 0, 1};
+   }
+   else
+   {
+      if (k <= 256) *s = {1, 64, 1, 0, 8};
+      else if (k <= 512) *s = {1, 64, 2, 0, 4};
+      else if (k <= 1024) *s = {1, 64, 4, 0, 2};
+      else *s = {1, 64, 8, 0, 1};
+   }
+   return FUSEDMM_SUCCESS_RETURN;
+}
+
+struct Launch {
+   int num_cu, blocks_per_cu;
+   hipStream_t stream;
+   hipEvent_t *ev;   // 4 events or nullptr
+};
+
+template <int V, int L, int R, bool EXACT, int OP, int U>
+int launch_instance(const Params<idx_t> &p, const Launch &l)
+{
+   // persistent grids: as many blocks as stay resident, each wave strides over rows
+   static int occ_rows = 0, occ_segs = 0;
+   if (occ_rows == 0)
+   {
+      FMM_HIP(hipOccupancyMaxActiveBlocksPerMultiprocessor(&occ_rows, rows_kernel<V, L, R, EXACT, OP, U, idx_t>, kBlockThreads, 0));
+      FMM_HIP(hipOccupancyMaxActiveBlocksPerMultiprocessor(&occ_segs, segments_kernel<V, L, R, EXACT, OP, U, idx_t>, kBlockThreads, 0));
+      if (occ_rows < 1) occ_rows = 1;
+      if (occ_segs < 1) occ_segs = 1;
+   }
+   const int64_t need = (p.m + kWavesPerBlock - 1) / kWavesPerBlock;
+   int64_t gr = (int64_t)l.num_cu * (l.blocks_per_cu > 0 ? l.blocks_per_cu : occ_rows);
+   if (gr > need) gr = need;
+   const int64_t gs = (int64_t)l.num_cu * (l.blocks_per_cu > 0 ? l.blocks_per_cu : occ_segs);
+   if (l.ev) FMM_HIP(hipEventRecord(l.ev[0], l.stream));
+   hipLaunchKernelGGL((rows_kernel<V, L, R, EXACT, OP, U, idx_t>), dim3((unsigned int)gr), dim3(kBlockThreads), 0, l.stream, p);
+   if (l.ev) FMM_HIP(hipEventRecord(l.ev[1], l.stream));
+   hipLaunchKernelGGL((segments_kernel<V, L, R, EXACT, OP, U, idx_t>), dim3((unsigned int)gs), dim3(kBlockThreads), 0, l.stream, p);
+   if (l.ev) FMM_HIP(hipEventRecord(l.ev[2], l.stream));
+   hipLaunchKernelGGL((merge_kernel<idx_t>), dim3((unsigned int)(l.num_cu * 2)), dim3(kBlockThreads), 0, l.stream, p, (int)(OP == OP_GENERIC));
+   if (l.ev) FMM_HIP(hipEventRecord(l.ev[3], l.stream));
+   return hip_status(hipGetLastError(), "kernel launch");
+}
+
+template <int OP>
+int launch_op(const Params<idx_t> &p, const Shape &s, const Launch &l)
+{
+#define FMM_CASE(V_, L_, R_, X_, U_) \
+   if (s.V == V_ && s.L == L_ && s.R == R_ && s.exact == X_) return launch_instance<V_, L_, R_, (X_ != 0), OP, U_>(p, l);
+   FMM_CASE(4, 8, 1, 1, 8)
+   FMM_CASE(4, 16, 1, 1, 8)
+   FMM_CASE(4, 32, 1, 1, 8)
+   FMM_CASE(4, 64, 1, 1, 8)
+   FMM_CASE(4, 64, 2, 1, 4)
+   FMM_CASE(4, 8, 1, 0, 8)
+   FMM_CASE(4, 16, 1, 0, 8)
+   FMM_CASE(4, 32, 1, 0, 8)
+   FMM_CASE(4, 64, 1, 0, 8)
+   FMM_CASE(4, 64, 2, 0, 4)
+   FMM_CASE(4, 64, 4, 0, 2)
+   FMM_CASE(4, 64, 8, 0, 1)
+   FMM_CASE(1, 64, 1, 0, 8)
+   FMM_CASE(1, 64, 2, 0, 4)
+   FMM_CASE(1, 64, 4, 0, 2)
+   FMM_CASE(1, 64, 8, 0, 1)
+#undef FMM_CASE
+   return FUSEDMM_FAIL_RETURN;
+}
+
+// ---- op tuple --------------------------------------------------------------------
+struct Plan {
+   int op;            // OP_*
+   bool opt_rule;     // optimised write-back rule (beta == 0 overwrites)
+   bool needs_sop;    // tuple uses SOP_UDEF
+   bool reads_x, reads_val;
+};
+
+// Stage validation in the order of reference fusedMM.c:610-628, then the
+// pattern match of :523-583.
+int make_plan(int32_t imsg, int opt_enabled, Plan *pl)
+{
+   const int vop = GET_VOP_FLAG(imsg), rop = GET_ROP_FLAG(imsg), sop = GET_SOP_FLAG(imsg),
+             vsc = GET_VSC_FLAG(imsg), aop = GET_AOP_FLAG(imsg);
+   if (imsg & ~0xFFFFF) { FMM_LOG("Unknown bits in imessage 0x%x", imsg); return FUSEDMM_FAIL_RETURN; }
+   if (vop == VOP_UDEF) { FMM_LOG("VOP_UDEF has no device implementation"); return FUSEDMM_UNDEFINED_USER_FUNCTION; }
+   if (vop < VOP_COPY_LHS || vop > VOP_MIN) { FMM_LOG("Unknown VOP Message"); return FUSEDMM_VOP_FAIL_RETURN; }
+   if (rop == ROP_UDEF) { FMM_LOG("ROP_UDEF has no device implementation"); return FUSEDMM_UNDEFINED_USER_FUNCTION; }
+   if (rop > ROP_NORMR) { FMM_LOG("Unknown ROP Message"); return FUSEDMM_ROP_FAIL_RETURN; }
+   if (!(sop == SOP_NOOP || sop == SOP_COPY || sop == SOP_UDEF)) { FMM_LOG("Unknown SOP Message"); return FUSEDMM_SOP_FAIL_RETURN; }
+   if (vsc == VSC_UDEF) { FMM_LOG("VSC_UDEF has no device implementation"); return FUSEDMM_UNDEFINED_USER_FUNCTION; }
+   if (vsc > VSC_ADD) { FMM_LOG("Unknown VSC Message"); return FUSEDMM_VSC_FAIL_RETURN; }
+   if (aop == AOP_UDEF) { FMM_LOG("AOP_UDEF has no device implementation"); return FUSEDMM_UNDEFINED_USER_FUNCTION; }
+   if (aop > AOP_MIN) { FMM_LOG("Unknown AOP Message"); return FUSEDMM_AOP_FAIL_RETURN; }
+
+   pl->needs_sop = (sop == SOP_UDEF);
+   pl->opt_rule = false;
+   pl->op = OP_GENERIC;
+   if (opt_enabled && vop == VOP_COPY_RHS && vsc != VSC_ADD && aop == AOP_ADD)
+   {
+      if (rop == ROP_NOOP && sop == SOP_NOOP && vsc == VSC_NOOP) pl->op = OP_GCN;
+      else if (rop == ROP_NOOP && sop == SOP_COPY && vsc == VSC_MUL) pl->op = OP_SPMM;
+      else if (rop == ROP_DOT && sop == SOP_UDEF && vsc == VSC_MUL) pl->op = OP_DOT;
+   }
+   if (opt_enabled && vop == VOP_SUBR && rop == ROP_NORMR && sop == SOP_UDEF && vsc == VSC_MUL && aop == AOP_ADD)
+      pl->op = OP_DIST;
+   pl->opt_rule = (pl->op != OP_GENERIC);
+   pl->reads_x = (pl->op == OP_DOT || pl->op == OP_DIST) ||
+                 (pl->op == OP_GENERIC && (vop != VOP_COPY_RHS || rop == ROP_DOT || rop == ROP_ADD_LHS || rop == ROP_NORML));
+   // the general pipeline seeds the scalar with val[j]; it matters only when no ROP overwrites it
+   pl->reads_val = (pl->op == OP_SPMM) || (pl->op == OP_GENERIC && rop == ROP_NOOP && vsc != VSC_NOOP);
+   return FUSEDMM_SUCCESS_RETURN;
+}
+
+struct Args {
+   int32_t imessage;
+   int64_t m, n, k, nnz;
+   const float *val;
+   const idx_t *indx, *pntrb, *pntre;
+   const float *x, *y;
+   float *z;
+   int64_t ldx, ldy, ldz;
+   float beta;
+};
+
+// Everything here is device memory.  Enqueues on `stream`, does not wait.
+int run_on_device(const Args &a, const Plan &pl, int sop_kind, hipStream_t stream)
+{
+   if (a.m <= 0) return FUSEDMM_SUCCESS_RETURN;
+   if (a.k < 1) return FUSEDMM_SUCCESS_RETURN;
+   if (a.k > kMaxK)
+   {
+      FMM_LOG("feature dimension k=%lld is beyond the supported maximum %d", (long long)a.k, kMaxK);
+      return FUSEDMM_FAIL_RETURN;
+   }
+   if (a.ldy < a.k || a.ldz < a.k || (pl.reads_x && a.ldx < a.k))
+   {
+      FMM_LOG("leading dimension smaller than k");
+      return FUSEDMM_FAIL_RETURN;
+   }
+   if (!a.indx || !a.pntrb || !a.pntre || !a.y || !a.z || (pl.reads_x && !a.x) || (pl.op == OP_SPMM && !a.val))
+   {
+      FMM_LOG("NULL operand");
+      return FUSEDMM_FAIL_RETURN;
+   }
+   DeviceState *d = nullptr;
+   int st = device_state(&d);
+   if (st) return st;
+
+   const bool vec_ok = (a.k % 4 == 0) && (a.ldy % 4 == 0) && (a.ldz % 4 == 0) && aligned16(a.y) && aligned16(a.z) &&
+                       (!pl.reads_x || ((a.ldx % 4 == 0) && aligned16(a.x)));
+   Shape sh;
+   st = pick_shape((int)a.k, vec_ok, &sh);
+   if (st) return st;
+
+   Params<idx_t> p;
+   memset(&p, 0, sizeof(p));
+   p.pntrb = a.pntrb; p.pntre = a.pntre; p.indx = a.indx;
+   p.val = pl.reads_val ? a.val : nullptr;
+   p.x = a.x; p.y = a.y; p.z = a.z;
+   p.m = a.m; p.ldx = a.ldx; p.ldy = a.ldy; p.ldz = a.ldz;
+   p.k = (int)a.k;
+   p.beta_zero = (pl.opt_rule && a.beta == 0.0f) ? 1 : 0;
+   p.sop_kind = sop_kind;
+   p.imessage = a.imessage;
+   p.sigmoid_table = d->sigmoid_table;
+
+   // heavy-row split: segments of about 256 KiB of gathered rows
+   int seg_len = g.seg_len > 0 ? g.seg_len : (int)(262144 / (4 * a.k));
+   if (seg_len < 64 && g.seg_len <= 0) seg_len = 64;
+   int64_t heavy_deg = g.heavy_deg > 0 ? g.heavy_deg : 2 * (int64_t)seg_len;
+   if (heavy_deg < seg_len) heavy_deg = seg_len;
+   p.seg_len = seg_len;
+   p.heavy_deg = heavy_deg;
+   p.kpad = (int)((a.k + 3) / 4 * 4);
+
+   // queue capacities from the caller's nnz when it is plausible; rows that do
+   // not fit are processed whole by the row kernel, so this is never a
+   // correctness question
+   int64_t nnz_hint = (a.nnz > 0 && a.nnz < ((int64_t)1 << 40)) ? a.nnz : (int64_t)1 << 26;
+   int64_t cap_seg = nnz_hint / seg_len * 3 / 2 + 1024;
+   int64_t cap_heavy = nnz_hint / heavy_deg + 1024;
+   const int64_t max_partial_bytes = (int64_t)8 << 30;
+   if (cap_seg * p.kpad * 4 > max_partial_bytes) cap_seg = max_partial_bytes / (p.kpad * 4);
+   if (cap_seg > 0x7FFFFFFF) cap_seg = 0x7FFFFFFF;
+   if (cap_heavy > 0x7FFFFFFF) cap_heavy = 0x7FFFFFFF;
+   st = grow(d->heavy, (size_t)cap_heavy * sizeof(HeavyRow)); if (st) return st;
+   st = grow(d->segs, (size_t)cap_seg * sizeof(SegDesc)); if (st) return st;
+   st = grow(d->partial, (size_t)cap_seg * p.kpad * sizeof(float)); if (st) return st;
+   p.ctr = d->ctr;
+   p.heavy = (HeavyRow *)d->heavy.ptr;
+   p.segs = (SegDesc *)d->segs.ptr;
+   p.partial = (float *)d->partial.ptr;
+   p.cap_heavy = (unsigned int)cap_heavy;
+   p.cap_seg = (unsigned int)cap_seg;
+
+   FMM_HIP(hipMemsetAsync(d->ctr, 0, sizeof(Counters), stream));
+
+   Launch l;
+   l.num_cu = d->num_cu;
+   l.blocks_per_cu = g.blocks_per_cu;
+   l.stream = stream;
+   l.ev = nullptr;
+   if (g.timing && g.timing_calls < kTimingSlots)
+   {
+      if (!d->ev_made)
+      {
+         for (int i = 0; i < kTimingSlots; i++)
+            for (int e = 0; e < 4; e++) FMM_HIP(hipEventCreate(&d->ev[i][e]));
+         d->ev_made = true;
+      }
+      l.ev = d->ev[g.timing_calls++];
+      FMM_HIP(hipGetDevice(&g.timing_dev));
+   }
+
+   switch (pl.op)
+   {
+      case OP_GCN: return launch_op<OP_GCN>(p, sh, l);
+      case OP_SPMM: return launch_op<OP_SPMM>(p, sh, l);
+      case OP_DOT: return launch_op<OP_DOT>(p, sh, l);
+      case OP_DIST: return launch_op<OP_DIST>(p, sh, l);
+      default: return launch_op<OP_GENERIC>(p, sh, l);
+   }
+}
+
+bool is_device_pointer(const void *p)
+{
+   if (!p) return false;
+   hipPointerAttribute_t attr;
+   hipError_t e = hipPointerGetAttributes(&attr, p);
+   if (e != hipSuccess)
+   {
+      (void)hipGetLastError();   // plain host memory: not an error for us
+      return false;
+   }
+   return attr.type == hipMemoryTypeDevice || attr.type == hipMemoryTypeManaged;
+}
+
+// Host-pointer mode: stage operands to the GPU, run, copy Z back.  Only the
+// first k columns of each Z row are written back, as the reference touches
+// nothing else.
+int run_staged(const Args &h, const Plan &pl, int sop_kind)
+{
+   if (h.m <= 0 || h.k < 1) return FUSEDMM_SUCCESS_RETURN;
+   if (h.n <= 0) { FMM_LOG("n (rows of Y) must be positive for host operands"); return FUSEDMM_FAIL_RETURN; }
+   DeviceState *d = nullptr;
+   int st = device_state(&d);
+   if (st) return st;
+   int64_t slots = 0;
+   for (int64_t i = 0; i < h.m; i++)
+      if ((int64_t)h.pntre[i] > slots) slots = (int64_t)h.pntre[i];
+   const bool need_val = pl.reads_val;
+   if (need_val && !h.val) { FMM_LOG("NULL operand"); return FUSEDMM_FAIL_RETURN; }
+   const size_t b_ptr = (size_t)h.m * sizeof(idx_t);
+   const size_t b_idx = (size_t)(slots > 0 ? slots : 1) * sizeof(idx_t);
+   const size_t b_val = (size_t)(slots > 0 ? slots : 1) * sizeof(float);
+   const size_t b_x = (size_t)h.m * (size_t)h.ldx * sizeof(float);
+   const size_t b_y = (size_t)h.n * (size_t)h.ldy * sizeof(float);
+   const size_t b_z = (size_t)h.m * (size_t)h.ldz * sizeof(float);
+   st = grow(d->stage[0], b_ptr); if (st) return st;
+   st = grow(d->stage[1], b_ptr); if (st) return st;
+   st = grow(d->stage[2], b_idx); if (st) return st;
+   if (need_val) { st = grow(d->stage[3], b_val); if (st) return st; }
+   if (pl.reads_x) { st = grow(d->stage[4], b_x); if (st) return st; }
+   st = grow(d->stage[5], b_y); if (st) return st;
+   st = grow(d->stage[6], b_z); if (st) return st;
+
+   hipStream_t s = 0;
+   FMM_HIP(hipMemcpyAsync(d->stage[0].ptr, h.pntrb, b_ptr, hipMemcpyHostToDevice, s));
+   FMM_HIP(hipMemcpyAsync(d->stage[1].ptr, h.pntre, b_ptr, hipMemcpyHostToDevice, s));
+   if (slots > 0) FMM_HIP(hipMemcpyAsync(d->stage[2].ptr, h.indx, (size_t)slots * sizeof(idx_t), hipMemcpyHostToDevice, s));
+   if (need_val && slots > 0) FMM_HIP(hipMemcpyAsync(d->stage[3].ptr, h.val, (size_t)slots * sizeof(float), hipMemcpyHostToDevice, s));
+   if (pl.reads_x) FMM_HIP(hipMemcpyAsync(d->stage[4].ptr, h.x, b_x, hipMemcpyHostToDevice, s));
+   FMM_HIP(hipMemcpyAsync(d->stage[5].ptr, h.y, b_y, hipMemcpyHostToDevice, s));
+   const bool overwrite = pl.opt_rule && h.beta == 0.0f;
+   if (!overwrite)
+      FMM_HIP(hipMemcpy2DAsync(d->stage[6].ptr, (size_t)h.ldz * 4, h.z, (size_t)h.ldz * 4, (size_t)h.k * 4, (size_t)h.m,
+                               hipMemcpyHostToDevice, s));
+   Args a = h;
+   a.pntrb = (const idx_t *)d->stage[0].ptr;
+   a.pntre = (const idx_t *)d->stage[1].ptr;
+   a.indx = (const idx_t *)d->stage[2].ptr;
+   a.val = need_val ? (const float *)d->stage[3].ptr : nullptr;
+   a.x = pl.reads_x ? (const float *)d->stage[4].ptr : nullptr;
+   a.y = (const float *)d->stage[5].ptr;
+   a.z = (float *)d->stage[6].ptr;
+   if (a.nnz <= 0 || a.nnz > slots) a.nnz = slots;
+   st = run_on_device(a, pl, sop_kind, s);
+   if (st) return st;
+   FMM_HIP(hipMemcpy2DAsync(h.z, (size_t)h.ldz * 4, d->stage[6].ptr, (size_t)h.ldz * 4, (size_t)h.k * 4, (size_t)h.m,
+                            hipMemcpyDeviceToHost, s));
+   FMM_HIP(hipStreamSynchronize(s));
+   return FUSEDMM_SUCCESS_RETURN;
+}
+
+int entry(const Args &a, bool async, hipStream_t stream)
+{
+   std::lock_guard<std::mutex> lock(g.mu);
+   read_env_once();
+   Plan pl;
+   int st = make_plan(a.imessage, g.opt, &pl);
+   if (st) return st;
+   int sop_kind = g.sop_kind;
+   if (pl.needs_sop && sop_kind == FUSEDMM_SOP_KIND_HOST)
+   {
+      FMM_LOG("SOP_UDEF with kind 'host' is not available in this build of the path; "
+              "select a device body with fusedMM_amd_set_sop_kind() or FUSEDMM_SOP_KIND");
+      return FUSEDMM_UNDEFINED_USER_FUNCTION;
+   }
+   if (async) return run_on_device(a, pl, sop_kind, stream);
+   if (is_device_pointer(a.z))
+   {
+      st = run_on_device(a, pl, sop_kind, 0);
+      if (st) return st;
+      return hip_status(hipStreamSynchronize(0), "hipStreamSynchronize");
+   }
+   return run_staged(a, pl, sop_kind);
+}
+
+}  // namespace
+
+// ---- exported C ABI -------------------------------------------------------------------
+extern "C" {
+
+int fusedMM_csr(const int32_t imessage, const INDEXTYPE m, const INDEXTYPE n, const INDEXTYPE k,
+                const VALUETYPE alpha, const INDEXTYPE nnz, const INDEXTYPE rows, const INDEXTYPE cols,
+                const VALUETYPE *val, const INDEXTYPE *indx, const INDEXTYPE *pntrb, const INDEXTYPE *pntre,
+                const VALUETYPE *x, const INDEXTYPE ldx, const VALUETYPE *y, const INDEXTYPE ldy,
+                const VALUETYPE beta, VALUETYPE *z, const INDEXTYPE ldz)
+{
+   (void)alpha; (void)rows; (void)cols;
+   Args a = {imessage, (int64_t)m, (int64_t)n, (int64_t)k, (int64_t)nnz, val, indx, pntrb, pntre, x, y, z,
+             (int64_t)ldx, (int64_t)ldy, (int64_t)ldz, beta};
+   return entry(a, false, 0);
+}
+
+int fusedMM_csr_stream(const int32_t imessage, const INDEXTYPE m, const INDEXTYPE n, const INDEXTYPE k,
+                       const VALUETYPE alpha, const INDEXTYPE nnz, const INDEXTYPE rows, const INDEXTYPE cols,
+                       const VALUETYPE *val, const INDEXTYPE *indx, const INDEXTYPE *pntrb, const INDEXTYPE *pntre,
+                       const VALUETYPE *x, const INDEXTYPE ldx, const VALUETYPE *y, const INDEXTYPE ldy,
+                       const VALUETYPE beta, VALUETYPE *z, const INDEXTYPE ldz, void *stream)
+{
+   (void)alpha; (void)rows; (void)cols;
+   Args a = {imessage, (int64_t)m, (int64_t)n, (int64_t)k, (int64_t)nnz, val, indx, pntrb, pntre, x, y, z,
+             (int64_t)ldx, (int64_t)ldy, (int64_t)ldz, beta};
+   return entry(a, true, (hipStream_t)stream);
+}
+
+void sgfusedMM_csr(const char tkern, const INDEXTYPE m, const INDEXTYPE n, const INDEXTYPE k, const float alpha,
+                   const INDEXTYPE nnz, const INDEXTYPE rows, const INDEXTYPE cols, const float *val,
+                   const INDEXTYPE *indx, const INDEXTYPE *pntrb, const INDEXTYPE *pntre, const float *a,
+                   const INDEXTYPE lda, const float *b, const INDEXTYPE ldb, const float beta, float *c,
+                   const INDEXTYPE ldc)
+{
+   int32_t imsg;
+   switch (tkern)
+   {
+      case 'g': imsg = VOP_COPY_RHS | ROP_NOOP | SOP_NOOP | VSC_NOOP | AOP_ADD; break;
+      case 'm': imsg = VOP_COPY_RHS | ROP_NOOP | SOP_COPY | VSC_MUL | AOP_ADD; break;
+      case 's': imsg = VOP_COPY_RHS | ROP_DOT | SOP_UDEF | VSC_MUL | AOP_ADD; break;
+      case 't': imsg = VOP_SUBR | ROP_NORMR | SOP_UDEF | VSC_MUL | AOP_ADD; break;
+      default:
+         fprintf(stderr, "unknown kernel type!\n");   // reference kernels.c:627-629 only prints
+         return;
+   }
+   (void)fusedMM_csr(imsg, m, n, k, alpha, nnz, rows, cols, val, indx, pntrb, pntre, a, lda, b, ldb, beta, c, ldc);
+}
+
+int fusedMM_amd_index_bytes(void) { return (int)sizeof(INDEXTYPE); }
+
+int fusedMM_amd_set_sop_kind(int kind)
+{
+   std::lock_guard<std::mutex> lock(g.mu);
+   read_env_once();
+   if (kind < FUSEDMM_SOP_KIND_HOST || kind > FUSEDMM_SOP_KIND_FA) return -2;
+   int prev = g.sop_kind;
+   g.sop_kind = kind;
+   return prev;
+}
+
+int fusedMM_amd_get_sop_kind(void)
+{
+   std::lock_guard<std::mutex> lock(g.mu);
+   read_env_once();
+   return g.sop_kind;
+}
+
+void fusedMM_amd_set_sop_callback(fusedMM_amd_sop_fn fn)
+{
+   std::lock_guard<std::mutex> lock(g.mu);
+   g.sop_fn = fn;
+}
+
+int fusedMM_amd_set_opt(int enable)
+{
+   std::lock_guard<std::mutex> lock(g.mu);
+   int prev = g.opt;
+   g.opt = enable ? 1 : 0;
+   return prev;
+}
+
+void fusedMM_amd_set_split(int64_t heavy_deg, int seg_len)
+{
+   std::lock_guard<std::mutex> lock(g.mu);
+   g.heavy_deg = heavy_deg > 0 ? heavy_deg : 0;
+   g.seg_len = seg_len > 0 ? seg_len : 0;
+}
+
+void fusedMM_amd_timing(int enable)
+{
+   std::lock_guard<std::mutex> lock(g.mu);
+   g.timing = enable != 0;
+   g.timing_calls = 0;
+}
+
+int fusedMM_amd_timing_summary(double *rows_ms, double *segments_ms, double *merge_ms)
+{
+   std::lock_guard<std::mutex> lock(g.mu);
+   double t[3] = {0, 0, 0};
+   int n = g.timing_calls;
+   if (n > 0)
+   {
+      DeviceState &d = g.dev[g.timing_dev];
+      if (hipEventSynchronize(d.ev[n - 1][3]) != hipSuccess) return -1;
+      for (int i = 0; i < n; i++)
+         for (int e = 0; e < 3; e++)
+         {
+            float ms = 0.f;
+            if (hipEventElapsedTime(&ms, d.ev[i][e], d.ev[i][e + 1]) != hipSuccess) return -1;
+            t[e] += ms;
+         }
+   }
+   if (rows_ms) *rows_ms = t[0];
+   if (segments_ms) *segments_ms = t[1];
+   if (merge_ms) *merge_ms = t[2];
+   return n;
+}
+
+int fusedMM_amd_last_split(unsigned int *heavy_rows, unsigned int *segments, unsigned int *overflow)
+{
+   std::lock_guard<std::mutex> lock(g.mu);
+   DeviceState *d = nullptr;
+   int st = device_state(&d);
+   if (st) return st;
+   Counters c;
+   FMM_HIP(hipDeviceSynchronize());
+   FMM_HIP(hipMemcpy(&c, d->ctr, sizeof(c), hipMemcpyDeviceToHost));
+   if (heavy_rows) *heavy_rows = c.n_heavy;
+   if (segments) *segments = c.n_seg;
+   if (overflow) *overflow = c.overflow;
+   return FUSEDMM_SUCCESS_RETURN;
+}
+
+void fusedMM_amd_finalize(void)
+{
+   std::lock_guard<std::mutex> lock(g.mu);
+   int cur = 0;
+   if (hipGetDevice(&cur) != hipSuccess) return;
+   for (int dev = 0; dev < kMaxDevices; dev++)
+   {
+      DeviceState &d = g.dev[dev];
+      if (!d.ready) continue;
+      if (hipSetDevice(dev) != hipSuccess) continue;
+      (void)hipDeviceSynchronize();
+      (void)hipFree(d.sigmoid_table);
+      (void)hipFree(d.ctr);
+      Buffer *bufs[] = {&d.heavy, &d.segs, &d.partial};
+      for (Buffer *b : bufs) { if (b->ptr) (void)hipFree(b->ptr); *b = Buffer(); }
+      for (Buffer &b : d.stage) { if (b.ptr) (void)hipFree(b.ptr); b = Buffer(); }
+      if (d.ev_made)
+         for (int i = 0; i < kTimingSlots; i++)
+            for (int e = 0; e < 4; e++) (void)hipEventDestroy(d.ev[i][e]);
+      d = DeviceState();
+   }
+   (void)hipSetDevice(cur);
+}
+
+}  // extern "C"

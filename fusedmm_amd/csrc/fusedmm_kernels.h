@@ -1,0 +1,684 @@
+// Device code for the fused SDDMM+SpMM path on gfx950 (wave64).
+//
+// One wavefront walks one CSR row (or one fixed-length edge segment of a heavy
+// row).  A wavefront is cut into S = 64/L sub-waves of L lanes; a sub-wave owns
+// one neighbour row Y[c] at a time, each lane holding R float4 slices of it, so
+// a gather is L coalesced 16-byte loads.  The X[i] slice and the Z accumulator
+// live in VGPRs for the whole row.  The per-edge reduction (ROP) is a DPP /
+// swizzle XOR butterfly over the L lanes, the scalar op (SOP) and the scaled
+// accumulate (MOP, AOP) happen in registers.
+//
+// Element e of a K-vector sits in lane (e/4) % L, register (e/4) / L,
+// component e % 4.  A lane reduces its own elements with a fused multiply-add
+// chain (register ascending, component ascending) and lanes are combined by XOR
+// offsets 1, 2, 4 ... L/2.  That order is part of the numerical contract: the
+// table sigmoid is discontinuous in the dot product, and the CPU oracle's
+// "wavefront order" mode reproduces exactly this sum.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace fmm {
+
+// ---- op-tuple nibbles (values of the public header) -------------------------
+enum : int {
+   kVopCopyLhs = 0x1, kVopCopyRhs = 0x2, kVopAdd = 0x3, kVopSubl = 0x4, kVopSubr = 0x5,
+   kVopMax = 0x6, kVopMin = 0x7,
+   kRopNoop = 0x00, kRopDot = 0x10, kRopAddLhs = 0x20, kRopAddRhs = 0x30, kRopNormL = 0x40,
+   kRopNormR = 0x50,
+   kSopNoop = 0x000, kSopCopy = 0x100, kSopUdef = 0xF00,
+   kVscNoop = 0x0000, kVscMul = 0x1000, kVscAdd = 0x2000,
+   kAopNoop = 0x00000, kAopAdd = 0x10000, kAopMax = 0x20000, kAopMin = 0x30000
+};
+
+// Pattern-matched kernels and the runtime-switched general one.
+enum : int { OP_GCN = 0, OP_SPMM = 1, OP_DOT = 2, OP_DIST = 3, OP_GENERIC = 4 };
+
+// Device-native bodies for SOP_UDEF (numbering shared with the public header).
+enum : int { SOP_IDENTITY = 0, SOP_SIGMOID = 1, SOP_TDIST = 2, SOP_FR = 3, SOP_LL = 4, SOP_FA = 5 };
+
+constexpr int kSigmoidTableSize = 2048;
+constexpr int kBlockThreads = 256;
+constexpr int kWavesPerBlock = kBlockThreads / 64;
+
+struct Counters {
+   unsigned int n_heavy;    // heavy rows queued by the row kernel
+   unsigned int n_seg;      // edge segments queued
+   unsigned int overflow;   // heavy rows that did not fit the queue (handled inline)
+   unsigned int pad;
+};
+
+struct HeavyRow {
+   int64_t row;
+   unsigned int seg_base;
+   unsigned int n_seg;
+};
+
+struct SegDesc {
+   int64_t row;
+   unsigned int seg;       // segment number inside the row
+   unsigned int pad;
+};
+
+template <typename IdxT>
+struct Params {
+   const IdxT *pntrb, *pntre, *indx;
+   const float *val;
+   const float *x, *y;
+   float *z;
+   int64_t m;
+   int64_t ldx, ldy, ldz;
+   int k;
+   int beta_zero;          // 1: overwrite Z, 0: accumulate into Z
+   int sop_kind;           // device SOP body for SOP_UDEF
+   int imessage;           // op tuple (read by OP_GENERIC only)
+   const float *sigmoid_table;
+   // heavy-row queue
+   int64_t heavy_deg;      // rows with more edges than this are split
+   int seg_len;            // edges per segment
+   Counters *ctr;
+   HeavyRow *heavy;
+   SegDesc *segs;
+   float *partial;         // [cap_seg][kpad]
+   unsigned int cap_heavy, cap_seg;
+   int kpad;
+};
+
+// ---- wave primitives --------------------------------------------------------
+__device__ __forceinline__ float as_f(int v) { return __builtin_bit_cast(float, v); }
+__device__ __forceinline__ int as_i(float v) { return __builtin_bit_cast(int, v); }
+
+template <int CTRL>
+__device__ __forceinline__ float dpp(float v)
+{
+   return as_f(__builtin_amdgcn_update_dpp(0, as_i(v), CTRL, 0xF, 0xF, false));
+}
+// value held by lane ^ 16 / lane ^ 32
+__device__ __forceinline__ float lane_xor16(float v) { return as_f(__builtin_amdgcn_ds_swizzle(as_i(v), 0x401F)); }
+
+// v[lane] + v[lane ^ 32]: one v_permlane32_swap gives both halves to every lane.
+__device__ __forceinline__ float add_xor32(float v)
+{
+   auto r = __builtin_amdgcn_permlane32_swap(as_i(v), as_i(v), false, false);
+   return as_f(r[0]) + as_f(r[1]);
+}
+
+// Sum over the L lanes of a sub-wave; every lane ends with the same bits.
+// After the quad steps all lanes of a quad agree, so the half-row and row
+// mirrors deliver exactly the value lane^4 / lane^8 holds.
+template <int L>
+__device__ __forceinline__ float subwave_sum(float v)
+{
+   if (L >= 2) v = v + dpp<0xB1>(v);   // quad_perm [1,0,3,2]  : lane ^ 1
+   if (L >= 4) v = v + dpp<0x4E>(v);   // quad_perm [2,3,0,1]  : lane ^ 2
+   if (L >= 8) v = v + dpp<0x141>(v);  // row_half_mirror      : lane ^ 4 (by value)
+   if (L >= 16) v = v + dpp<0x140>(v); // row_mirror           : lane ^ 8 (by value)
+   if (L >= 32) v = v + lane_xor16(v);
+   if (L >= 64) v = add_xor32(v);
+   return v;
+}
+
+// Combine the S = 64/L sub-wave accumulators (same element slice, different
+// edges).  Offsets L, 2L .. 32 are true lane XORs (row_ror:8 == lane ^ 8).
+template <int L>
+__device__ __forceinline__ float cross_subwave_sum(float v)
+{
+   static_assert(L >= 8, "sub-waves narrower than 8 lanes are not used");
+   if (L <= 8) v = v + dpp<0x128>(v);  // row_ror:8
+   if (L <= 16) v = v + lane_xor16(v);
+   if (L <= 32) v = add_xor32(v);
+   return v;
+}
+template <int L>
+__device__ __forceinline__ float cross_subwave_max(float v)
+{
+   if (L <= 8) v = fmaxf(v, dpp<0x128>(v));
+   if (L <= 16) v = fmaxf(v, lane_xor16(v));
+   if (L <= 32) v = fmaxf(v, __shfl_xor(v, 32, 64));
+   return v;
+}
+template <int L>
+__device__ __forceinline__ float cross_subwave_min(float v)
+{
+   if (L <= 8) v = fminf(v, dpp<0x128>(v));
+   if (L <= 16) v = fminf(v, lane_xor16(v));
+   if (L <= 32) v = fminf(v, __shfl_xor(v, 32, 64));
+   return v;
+}
+
+template <typename T>
+__device__ __forceinline__ T wave_uniform(T v);
+template <>
+__device__ __forceinline__ int32_t wave_uniform<int32_t>(int32_t v) { return __builtin_amdgcn_readfirstlane(v); }
+template <>
+__device__ __forceinline__ int64_t wave_uniform<int64_t>(int64_t v)
+{
+   int lo = __builtin_amdgcn_readfirstlane((int)(v & 0xFFFFFFFFll));
+   int hi = __builtin_amdgcn_readfirstlane((int)(v >> 32));
+   return ((int64_t)hi << 32) | (uint32_t)lo;
+}
+
+// ---- SOP bodies ---------------------------------------------------------------
+// Same expressions, in the same precision, as the SOP_UDEF_FUNC bodies of the
+// reference's tester (test/fusedMMtime.cpp:606-660): constants there are double
+// literals, so the arithmetic is done in double and rounded once to float.
+__device__ __forceinline__ float sop_eval(int kind, float s, const float *tab)
+{
+   switch (kind)
+   {
+      case SOP_SIGMOID:
+      {
+         // floor-indexed 2048-entry table on [-5,5] (test/fusedMMtime.cpp:128-130, 606-611);
+         // s == 5 exactly would index one past the end there: clamp to the last entry.
+         float t;
+         if (s > 5.0f) t = 1.0f;
+         else if (s < -5.0f) t = 0.0f;
+         else
+         {
+            int idx = (int)(((double)s + 5.0) * 2048.0 / 10.0);
+            idx = idx > kSigmoidTableSize - 1 ? kSigmoidTableSize - 1 : idx;
+            t = tab[idx];
+         }
+         return 1.0f - t;   // exact in double for table values, so one rounding either way
+      }
+      case SOP_TDIST:
+      {
+         float t = (float)(-2.0 / (1.0 + (double)s));
+         t = t > 5.0f ? 5.0f : t;
+         t = t < -5.0f ? -5.0f : t;
+         return t;
+      }
+      case SOP_FR:
+         return (float)(1.0 + 1.0 / (double)s);
+      case SOP_LL:
+         return log2f(1.0f + sqrtf(s));
+      case SOP_FA:
+         return (float)((double)sqrtf(s) + 1.0 / (double)s);
+      default:
+         return s;
+   }
+}
+
+__device__ __forceinline__ float4 ld4(const float *p) { return *reinterpret_cast<const float4 *>(p); }
+__device__ __forceinline__ void st4(float *p, float4 v) { *reinterpret_cast<float4 *>(p) = v; }
+__device__ __forceinline__ float4 zero4() { return make_float4(0.f, 0.f, 0.f, 0.f); }
+
+// One row slice per lane: R float4 registers.
+template <int R>
+struct Slice {
+   float4 v[R];
+};
+
+// V == 4: lane sl holds elements 4*(r*L+sl) .. +3 in register r (16-byte accesses).
+// V == 1: rows that are not 16-byte aligned (K or a leading dimension not a
+// multiple of 4, or an unaligned base): component c of register r holds
+// element (4r+c)*L + sl, loaded and stored 4 bytes at a time.
+template <int V, int L, int R, bool EXACT>
+__device__ __forceinline__ void load_slice(Slice<R> &s, const float *row, int sl, int k)
+{
+#pragma unroll
+   for (int r = 0; r < R; r++)
+   {
+      if (V == 4)
+      {
+         const int e0 = 4 * (r * L + sl);
+         if (EXACT || e0 < k) s.v[r] = ld4(row + e0);
+         else s.v[r] = zero4();
+      }
+      else
+      {
+         const int e0 = (4 * r) * L + sl;
+         s.v[r].x = (e0 < k) ? row[e0] : 0.0f;
+         s.v[r].y = (e0 + L < k) ? row[e0 + L] : 0.0f;
+         s.v[r].z = (e0 + 2 * L < k) ? row[e0 + 2 * L] : 0.0f;
+         s.v[r].w = (e0 + 3 * L < k) ? row[e0 + 3 * L] : 0.0f;
+      }
+   }
+}
+
+template <int V, int L, int R, bool EXACT>
+__device__ __forceinline__ void store_slice(float *row, const Slice<R> &s, int sl, int k)
+{
+#pragma unroll
+   for (int r = 0; r < R; r++)
+   {
+      if (V == 4)
+      {
+         const int e0 = 4 * (r * L + sl);
+         if (EXACT || e0 < k) st4(row + e0, s.v[r]);
+      }
+      else
+      {
+         const int e0 = (4 * r) * L + sl;
+         if (e0 < k) row[e0] = s.v[r].x;
+         if (e0 + L < k) row[e0 + L] = s.v[r].y;
+         if (e0 + 2 * L < k) row[e0 + 2 * L] = s.v[r].z;
+         if (e0 + 3 * L < k) row[e0 + 3 * L] = s.v[r].w;
+      }
+   }
+}
+
+template <int L, int R>
+__device__ __forceinline__ float dot_slices(const Slice<R> &a, const Slice<R> &b)
+{
+   float p = 0.0f;
+#pragma unroll
+   for (int r = 0; r < R; r++)
+   {
+      p = __builtin_fmaf(a.v[r].x, b.v[r].x, p);
+      p = __builtin_fmaf(a.v[r].y, b.v[r].y, p);
+      p = __builtin_fmaf(a.v[r].z, b.v[r].z, p);
+      p = __builtin_fmaf(a.v[r].w, b.v[r].w, p);
+   }
+   return subwave_sum<L>(p);
+}
+
+template <int L, int R>
+__device__ __forceinline__ float sum_slice(const Slice<R> &a)
+{
+   float p = 0.0f;
+#pragma unroll
+   for (int r = 0; r < R; r++) p = ((((p + a.v[r].x) + a.v[r].y) + a.v[r].z) + a.v[r].w);
+   return subwave_sum<L>(p);
+}
+
+// acc = fma(d, t, acc) over a slice
+template <int R>
+__device__ __forceinline__ void axpy_slice(Slice<R> &acc, float d, const Slice<R> &t)
+{
+#pragma unroll
+   for (int r = 0; r < R; r++)
+   {
+      acc.v[r].x = __builtin_fmaf(d, t.v[r].x, acc.v[r].x);
+      acc.v[r].y = __builtin_fmaf(d, t.v[r].y, acc.v[r].y);
+      acc.v[r].z = __builtin_fmaf(d, t.v[r].z, acc.v[r].z);
+      acc.v[r].w = __builtin_fmaf(d, t.v[r].w, acc.v[r].w);
+   }
+}
+
+template <int R>
+__device__ __forceinline__ void sub_slices(Slice<R> &t, const Slice<R> &a, const Slice<R> &b)
+{
+#pragma unroll
+   for (int r = 0; r < R; r++)
+   {
+      t.v[r].x = a.v[r].x - b.v[r].x;
+      t.v[r].y = a.v[r].y - b.v[r].y;
+      t.v[r].z = a.v[r].z - b.v[r].z;
+      t.v[r].w = a.v[r].w - b.v[r].w;
+   }
+}
+
+template <class F, int R>
+__device__ __forceinline__ void map2(Slice<R> &o, const Slice<R> &a, const Slice<R> &b, F f)
+{
+#pragma unroll
+   for (int r = 0; r < R; r++)
+   {
+      o.v[r].x = f(a.v[r].x, b.v[r].x);
+      o.v[r].y = f(a.v[r].y, b.v[r].y);
+      o.v[r].z = f(a.v[r].z, b.v[r].z);
+      o.v[r].w = f(a.v[r].w, b.v[r].w);
+   }
+}
+
+// Identity element of the accumulate stage (what a sub-wave that did not load
+// Z starts from).
+__device__ __forceinline__ float aop_identity(int aop)
+{
+   if (aop == kAopMax) return -__builtin_inff();
+   if (aop == kAopMin) return __builtin_inff();
+   return 0.0f;
+}
+
+// The per-edge pipeline: T = VOP(x, y); s = ROP(x, T); d = SOP(s); T = MOP(d, T);
+// acc = AOP(acc, T).  `xs` is the X[i] slice, `ys` the gathered Y[c] slice.
+template <int L, int R, int OP>
+__device__ __forceinline__ void edge_step(Slice<R> &acc, const Slice<R> &xs, const Slice<R> &ys,
+                                          float edge_val, int sop_kind, int imsg, const float *tab)
+{
+   if (OP == OP_GCN)
+   {
+#pragma unroll
+      for (int r = 0; r < R; r++)
+      {
+         acc.v[r].x += ys.v[r].x;
+         acc.v[r].y += ys.v[r].y;
+         acc.v[r].z += ys.v[r].z;
+         acc.v[r].w += ys.v[r].w;
+      }
+   }
+   else if (OP == OP_SPMM)
+   {
+      axpy_slice<R>(acc, edge_val, ys);
+   }
+   else if (OP == OP_DOT)
+   {
+      const float s = dot_slices<L, R>(xs, ys);
+      const float d = sop_eval(sop_kind, s, tab);
+      axpy_slice<R>(acc, d, ys);
+   }
+   else if (OP == OP_DIST)
+   {
+      Slice<R> t;
+      sub_slices<R>(t, xs, ys);
+      const float s = dot_slices<L, R>(t, t);
+      const float d = sop_eval(sop_kind, s, tab);
+      axpy_slice<R>(acc, d, t);
+   }
+   else
+   {
+      const int vop = imsg & 0xF, rop = imsg & 0xF0, sop = imsg & 0xF00, vsc = imsg & 0xF000,
+                aop = imsg & 0xF0000;
+      Slice<R> t;
+      switch (vop)
+      {
+         case kVopCopyLhs: t = xs; break;
+         case kVopCopyRhs: t = ys; break;
+         case kVopAdd: map2(t, xs, ys, [](float a, float b) { return a + b; }); break;
+         case kVopSubl: map2(t, xs, ys, [](float a, float b) { return -a + b; }); break;
+         case kVopSubr: map2(t, xs, ys, [](float a, float b) { return a - b; }); break;
+         case kVopMax: map2(t, xs, ys, [](float a, float b) { return a > b ? a : b; }); break;
+         default: map2(t, xs, ys, [](float a, float b) { return a < b ? a : b; }); break;
+      }
+      float scal = edge_val;
+      switch (rop)
+      {
+         case kRopDot: scal = dot_slices<L, R>(xs, t); break;
+         case kRopAddLhs: scal = sum_slice<L, R>(xs); break;
+         case kRopAddRhs: scal = sum_slice<L, R>(t); break;
+         case kRopNormL: scal = dot_slices<L, R>(xs, xs); break;
+         case kRopNormR: scal = dot_slices<L, R>(t, t); break;
+         default: break;
+      }
+      const float d = (sop == kSopUdef) ? sop_eval(sop_kind, scal, tab) : scal;
+      if (vsc == kVscMul)
+      {
+#pragma unroll
+         for (int r = 0; r < R; r++)
+         {
+            t.v[r].x = d * t.v[r].x; t.v[r].y = d * t.v[r].y;
+            t.v[r].z = d * t.v[r].z; t.v[r].w = d * t.v[r].w;
+         }
+      }
+      else if (vsc == kVscAdd)
+      {
+#pragma unroll
+         for (int r = 0; r < R; r++)
+         {
+            t.v[r].x = d + t.v[r].x; t.v[r].y = d + t.v[r].y;
+            t.v[r].z = d + t.v[r].z; t.v[r].w = d + t.v[r].w;
+         }
+      }
+      if (aop == kAopAdd) map2(acc, acc, t, [](float a, float b) { return a + b; });
+      else if (aop == kAopMax) map2(acc, acc, t, [](float a, float b) { return a > b ? a : b; });
+      else if (aop == kAopMin) map2(acc, acc, t, [](float a, float b) { return a < b ? a : b; });
+   }
+}
+
+// Edges [jb, je) of one row, dealt round-robin to the sub-waves, U gathers in
+// flight per sub-wave.  All lanes of the wave call this with the same jb, je.
+template <int V, int L, int R, bool EXACT, int OP, int U, typename IdxT>
+__device__ __forceinline__ void walk_edges(Slice<R> &acc, const Slice<R> &xs, const Params<IdxT> &p,
+                                           IdxT jb, IdxT je, int sub, int sl, const float *tab)
+{
+   constexpr int S = 64 / L;
+   for (IdxT j0 = jb; j0 < je; j0 += S * U)
+   {
+      IdxT col[U];
+      float ev[U];
+      Slice<R> ys[U];
+#pragma unroll
+      for (int u = 0; u < U; u++)
+      {
+         const IdxT j = j0 + sub + u * S;
+         col[u] = -1;
+         ev[u] = 0.0f;
+         if (j < je)
+         {
+            col[u] = p.indx[j];
+            if (OP == OP_SPMM || OP == OP_GENERIC) ev[u] = p.val ? p.val[j] : 0.0f;
+         }
+      }
+#pragma unroll
+      for (int u = 0; u < U; u++)
+         if (col[u] >= 0) load_slice<V, L, R, EXACT>(ys[u], p.y + (int64_t)col[u] * p.ldy, sl, p.k);
+#pragma unroll
+      for (int u = 0; u < U; u++)
+         if (col[u] >= 0) edge_step<L, R, OP>(acc, xs, ys[u], ev[u], p.sop_kind, p.imessage, tab);
+   }
+}
+
+template <int L, int R, int OP>
+__device__ __forceinline__ void merge_subwaves(Slice<R> &acc, int imsg)
+{
+   if (L == 64) return;
+   const int aop = imsg & 0xF0000;
+#pragma unroll
+   for (int r = 0; r < R; r++)
+   {
+      if (OP == OP_GENERIC && aop == kAopMax)
+      {
+         acc.v[r].x = cross_subwave_max<L>(acc.v[r].x); acc.v[r].y = cross_subwave_max<L>(acc.v[r].y);
+         acc.v[r].z = cross_subwave_max<L>(acc.v[r].z); acc.v[r].w = cross_subwave_max<L>(acc.v[r].w);
+      }
+      else if (OP == OP_GENERIC && aop == kAopMin)
+      {
+         acc.v[r].x = cross_subwave_min<L>(acc.v[r].x); acc.v[r].y = cross_subwave_min<L>(acc.v[r].y);
+         acc.v[r].z = cross_subwave_min<L>(acc.v[r].z); acc.v[r].w = cross_subwave_min<L>(acc.v[r].w);
+      }
+      else
+      {
+         acc.v[r].x = cross_subwave_sum<L>(acc.v[r].x); acc.v[r].y = cross_subwave_sum<L>(acc.v[r].y);
+         acc.v[r].z = cross_subwave_sum<L>(acc.v[r].z); acc.v[r].w = cross_subwave_sum<L>(acc.v[r].w);
+      }
+   }
+}
+
+template <int OP>
+__device__ __forceinline__ bool op_reads_x(int imsg)
+{
+   if (OP == OP_DOT || OP == OP_DIST) return true;
+   if (OP == OP_GENERIC)
+   {
+      const int vop = imsg & 0xF, rop = imsg & 0xF0;
+      return vop != kVopCopyRhs || rop == kRopDot || rop == kRopAddLhs || rop == kRopNormL;
+   }
+   return false;
+}
+
+__device__ __forceinline__ const float *stage_table(const float *gtab, float *lds, bool need)
+{
+   if (!need) return gtab;
+   for (int i = threadIdx.x; i < kSigmoidTableSize; i += kBlockThreads) lds[i] = gtab[i];
+   __syncthreads();
+   return lds;
+}
+
+// ---- kernel 1: one wavefront per row, heavy rows queued -------------------------
+template <int V, int L, int R, bool EXACT, int OP, int U, typename IdxT>
+__global__ __launch_bounds__(kBlockThreads) void rows_kernel(const Params<IdxT> p)
+{
+   constexpr int S = 64 / L;
+   __shared__ float lds_tab[(OP >= OP_DOT) ? kSigmoidTableSize : 1];
+   const bool uses_sop = (OP == OP_DOT || OP == OP_DIST || (OP == OP_GENERIC && (p.imessage & 0xF00) == kSopUdef));
+   const float *tab = stage_table(p.sigmoid_table, lds_tab, (OP >= OP_DOT) && uses_sop && p.sop_kind == SOP_SIGMOID);
+
+   const int lane = threadIdx.x & 63;
+   const int sub = lane / L, sl = lane % L;
+   const int64_t wave0 = (int64_t)blockIdx.x * kWavesPerBlock + (threadIdx.x >> 6);
+   const int64_t nwaves = (int64_t)gridDim.x * kWavesPerBlock;
+   const bool reads_x = op_reads_x<OP>(p.imessage);
+   const int aop = p.imessage & 0xF0000;
+   const bool generic = (OP == OP_GENERIC);
+
+   for (int64_t row = wave0; row < p.m; row += nwaves)
+   {
+      const IdxT jb = wave_uniform<IdxT>(p.pntrb[row]);
+      const IdxT je = wave_uniform<IdxT>(p.pntre[row]);
+      const int64_t deg = (int64_t)je - (int64_t)jb;
+
+      if (deg > p.heavy_deg)
+      {
+         // queue the row for the segment kernel; if the queue is full, fall through
+         unsigned int nseg = (unsigned int)((deg + p.seg_len - 1) / p.seg_len);
+         unsigned int slot = 0, base = 0;
+         if (lane == 0)
+         {
+            slot = atomicAdd(&p.ctr->n_heavy, 1u);
+            base = atomicAdd(&p.ctr->n_seg, nseg);
+         }
+         slot = (unsigned int)__builtin_amdgcn_readfirstlane((int)slot);
+         base = (unsigned int)__builtin_amdgcn_readfirstlane((int)base);
+         const bool fits = slot < p.cap_heavy && (uint64_t)base + nseg <= (uint64_t)p.cap_seg;
+         if (fits)
+         {
+            if (lane == 0) p.heavy[slot] = HeavyRow{row, base, nseg};
+            for (unsigned int s = lane; s < nseg; s += 64) p.segs[base + s] = SegDesc{row, s, 0u};
+            continue;
+         }
+         // mark the slot unused (the merge kernel skips n_seg == 0) and do the row here
+         if (lane == 0)
+         {
+            if (slot < p.cap_heavy) p.heavy[slot] = HeavyRow{row, 0u, 0u};
+            atomicAdd(&p.ctr->overflow, 1u);
+         }
+         // every queue entry below the cap has exactly one writer: poison ours
+         for (uint64_t s = (uint64_t)base + lane; s < (uint64_t)base + nseg && s < (uint64_t)p.cap_seg; s += 64)
+            p.segs[s] = SegDesc{-1, 0u, 0u};
+      }
+
+      Slice<R> xs, acc;
+      if (reads_x) load_slice<V, L, R, EXACT>(xs, p.x + row * p.ldx, sl, p.k);
+      else
+      {
+#pragma unroll
+         for (int r = 0; r < R; r++) xs.v[r] = zero4();
+      }
+      float *zrow = p.z + row * p.ldz;
+      if (generic)
+      {
+         // general semantics: fold the edges into the caller's Z with AOP
+         if (aop == kAopNoop) continue;
+         if (sub == 0) load_slice<V, L, R, EXACT>(acc, zrow, sl, p.k);
+         else
+         {
+            const float id = aop_identity(aop);
+#pragma unroll
+            for (int r = 0; r < R; r++) acc.v[r] = make_float4(id, id, id, id);
+         }
+      }
+      else
+      {
+#pragma unroll
+         for (int r = 0; r < R; r++) acc.v[r] = zero4();
+      }
+
+      walk_edges<V, L, R, EXACT, OP, U, IdxT>(acc, xs, p, jb, je, sub, sl, tab);
+      merge_subwaves<L, R, OP>(acc, p.imessage);
+
+      if (sub == 0)
+      {
+         if (!generic && !p.beta_zero)
+         {
+            Slice<R> zin;
+            load_slice<V, L, R, EXACT>(zin, zrow, sl, p.k);
+            map2(acc, zin, acc, [](float a, float b) { return a + b; });
+         }
+         store_slice<V, L, R, EXACT>(zrow, acc, sl, p.k);
+      }
+   }
+}
+
+// ---- kernel 2: one wavefront per queued edge segment -> partial Z -----------------
+template <int V, int L, int R, bool EXACT, int OP, int U, typename IdxT>
+__global__ __launch_bounds__(kBlockThreads) void segments_kernel(const Params<IdxT> p)
+{
+   __shared__ float lds_tab[(OP >= OP_DOT) ? kSigmoidTableSize : 1];
+   unsigned int nseg = p.ctr->n_seg;
+   if (nseg > p.cap_seg) nseg = p.cap_seg;   // rows beyond the cap were done inline
+   if (nseg == 0) return;
+   const bool uses_sop = (OP == OP_DOT || OP == OP_DIST || (OP == OP_GENERIC && (p.imessage & 0xF00) == kSopUdef));
+   const float *tab = stage_table(p.sigmoid_table, lds_tab, (OP >= OP_DOT) && uses_sop && p.sop_kind == SOP_SIGMOID);
+
+   const int lane = threadIdx.x & 63;
+   const int sub = lane / L, sl = lane % L;
+   const int64_t wave0 = (int64_t)blockIdx.x * kWavesPerBlock + (threadIdx.x >> 6);
+   const int64_t nwaves = (int64_t)gridDim.x * kWavesPerBlock;
+   const bool reads_x = op_reads_x<OP>(p.imessage);
+   const int aop = p.imessage & 0xF0000;
+
+   for (int64_t q = wave0; q < (int64_t)nseg; q += nwaves)
+   {
+      const SegDesc sd = p.segs[q];
+      const int64_t row = wave_uniform<int64_t>(sd.row);
+      const unsigned int seg = (unsigned int)__builtin_amdgcn_readfirstlane((int)sd.seg);
+      if (row < 0) continue;   // slot of a row that was handled inline
+      const IdxT rb = wave_uniform<IdxT>(p.pntrb[row]);
+      const IdxT re = wave_uniform<IdxT>(p.pntre[row]);
+      const IdxT jb = rb + (IdxT)seg * (IdxT)p.seg_len;
+      IdxT je = jb + (IdxT)p.seg_len;
+      if (je > re) je = re;
+
+      Slice<R> xs, acc;
+      if (reads_x) load_slice<V, L, R, EXACT>(xs, p.x + row * p.ldx, sl, p.k);
+      else
+      {
+#pragma unroll
+         for (int r = 0; r < R; r++) xs.v[r] = zero4();
+      }
+      const float id = (OP == OP_GENERIC) ? aop_identity(aop) : 0.0f;
+#pragma unroll
+      for (int r = 0; r < R; r++) acc.v[r] = make_float4(id, id, id, id);
+
+      walk_edges<V, L, R, EXACT, OP, U, IdxT>(acc, xs, p, jb, je, sub, sl, tab);
+      merge_subwaves<L, R, OP>(acc, p.imessage);
+
+      if (sub == 0) store_slice<V, L, R, EXACT>(p.partial + (int64_t)q * p.kpad, acc, sl, p.k);
+   }
+}
+
+// ---- kernel 3: fold the partials of each heavy row, in segment order ----------------
+// One block per heavy row; thread t owns elements t, t+256, ...; the fold over
+// segments is sequential and therefore the same on every run.
+template <typename IdxT>
+__global__ __launch_bounds__(kBlockThreads) void merge_kernel(const Params<IdxT> p, int generic)
+{
+   unsigned int nheavy = p.ctr->n_heavy;
+   if (nheavy > p.cap_heavy) nheavy = p.cap_heavy;
+   const int aop = p.imessage & 0xF0000;
+   for (unsigned int h = blockIdx.x; h < nheavy; h += gridDim.x)
+   {
+      const HeavyRow hr = p.heavy[h];
+      if (hr.n_seg == 0) continue;
+      float *zrow = p.z + hr.row * p.ldz;
+      for (int e = threadIdx.x; e < p.k; e += kBlockThreads)
+      {
+         const float *pp = p.partial + (int64_t)hr.seg_base * p.kpad + e;
+         float a;
+         if (generic) a = zrow[e];
+         else a = 0.0f;
+         if (generic && aop == kAopMax)
+            for (unsigned int s = 0; s < hr.n_seg; s++) a = fmaxf(a, pp[(int64_t)s * p.kpad]);
+         else if (generic && aop == kAopMin)
+            for (unsigned int s = 0; s < hr.n_seg; s++) a = fminf(a, pp[(int64_t)s * p.kpad]);
+         else
+         {
+            unsigned int s = 0;
+            for (; s + 8 <= hr.n_seg; s += 8)
+            {
+               float v[8];
+#pragma unroll
+               for (int u = 0; u < 8; u++) v[u] = pp[(int64_t)(s + u) * p.kpad];
+#pragma unroll
+               for (int u = 0; u < 8; u++) a += v[u];
+            }
+            for (; s < hr.n_seg; s++) a += pp[(int64_t)s * p.kpad];
+         }
+         if (!generic && !p.beta_zero) a = zrow[e] + a;
+         zrow[e] = a;
+      }
+   }
+}
+
+}  // namespace fmm

@@ -1,0 +1,113 @@
+/*
+ * fusedmm_amd.h -- entry points of libfusedmm_amd_i{32,64}.so beyond the
+ * reference's fusedMM.h.  Plain C ABI: pointers, sizes and ints only.
+ * Define INDEXTYPE / VALUETYPE before including, as for fusedMM.h.
+ */
+#ifndef FUSEDMM_AMD_H
+#define FUSEDMM_AMD_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/*
+ * Device-native bodies for the SOP_UDEF stage.  They restate, expression for
+ * expression, the SOP_UDEF_FUNC bodies the reference's tester compiles, one
+ * per executable (reference test/fusedMMtime.cpp:626-674).
+ */
+#define FUSEDMM_SOP_KIND_HOST     (-1) /* call the host symbol SOP_UDEF_FUNC per edge (three passes) */
+#define FUSEDMM_SOP_KIND_IDENTITY   0  /* d = s                          (:668-673) */
+#define FUSEDMM_SOP_KIND_SIGMOID    1  /* d = 1 - table_sigmoid(s)       (:606-611, 628-632) */
+#define FUSEDMM_SOP_KIND_TDIST      2  /* d = clamp(-2/(1+s), -5, 5)     (:613-618, 642-646) */
+#define FUSEDMM_SOP_KIND_FR         3  /* d = 1 + 1/s                    (:635-639) */
+#define FUSEDMM_SOP_KIND_LL         4  /* d = log2(1 + sqrt(s))          (:649-653) */
+#define FUSEDMM_SOP_KIND_FA         5  /* d = sqrt(s) + 1/s              (:656-660) */
+
+/*
+ * Choose what SOP_UDEF means for later fusedMM_csr calls of this process.
+ * Replaces the reference's link-time choice of a SOP_UDEF_FUNC body
+ * (kernels/CONFIG/make.base:339-345 builds one executable per -D<KIND>_UDEF).
+ * Returns the previous kind, or -2 for an unknown kind.  The initial kind comes
+ * from the environment variable FUSEDMM_SOP_KIND (host, identity, sigmoid,
+ * tdist, fr, ll, fa) and is "host" when that is unset.
+ */
+int fusedMM_amd_set_sop_kind(int kind);
+int fusedMM_amd_get_sop_kind(void);
+
+/*
+ * Register the host SOP function used by FUSEDMM_SOP_KIND_HOST.  When never
+ * called, the library looks up the symbol SOP_UDEF_FUNC in the process, which
+ * is how the reference binds it (fusedMM.h:139; genkern.base:487, 554).
+ */
+typedef int (*fusedMM_amd_sop_fn)(VALUETYPE val, VALUETYPE *out);
+void fusedMM_amd_set_sop_callback(fusedMM_amd_sop_fn fn);
+
+/*
+ * fusedMM_csr on a caller-supplied HIP stream: every pointer is device memory,
+ * work is enqueued on `stream` (a hipStream_t; NULL is the default stream) and
+ * the call returns without waiting.  No counterpart in the reference; it is what
+ * a framework that already keeps its tensors on the GPU binds (the reference's
+ * CMakeLists.txt:1-14 packages fusedMM_csr for DGL).  FUSEDMM_SOP_KIND_HOST is
+ * not available here (it needs the host between passes): returns
+ * FUSEDMM_UNDEFINED_USER_FUNCTION.
+ */
+int fusedMM_csr_stream
+(
+   const int32_t imessage, const INDEXTYPE m, const INDEXTYPE n, const INDEXTYPE k,
+   const VALUETYPE alpha, const INDEXTYPE nnz, const INDEXTYPE rows, const INDEXTYPE cols,
+   const VALUETYPE *val, const INDEXTYPE *indx, const INDEXTYPE *pntrb, const INDEXTYPE *pntre,
+   const VALUETYPE *x, const INDEXTYPE ldx, const VALUETYPE *y, const INDEXTYPE ldy,
+   const VALUETYPE beta, VALUETYPE *z, const INDEXTYPE ldz, void *stream
+);
+
+/*
+ * The reference's second-level entry (kernels/include/kernels.h:32-37,
+ * kernels/src/kernels.c:456-631): tkern 'g' gcn, 'm' spmm, 's' sigmoid,
+ * 't' t-dist/FR.  Same pointer rules as fusedMM_csr.
+ */
+void sgfusedMM_csr
+(
+   const char tkern, const INDEXTYPE m, const INDEXTYPE n, const INDEXTYPE k,
+   const float alpha, const INDEXTYPE nnz, const INDEXTYPE rows, const INDEXTYPE cols,
+   const float *val, const INDEXTYPE *indx, const INDEXTYPE *pntrb, const INDEXTYPE *pntre,
+   const float *a, const INDEXTYPE lda, const float *b, const INDEXTYPE ldb,
+   const float beta, float *c, const INDEXTYPE ldc
+);
+
+/* sizeof(INDEXTYPE) this library was built for (4 or 8). */
+int fusedMM_amd_index_bytes(void);
+
+/* 1: pattern-matched tuples use the optimised kernels' write-back rule
+ * (default, the reference's ENABLE_OPT_FUSEDMM build, fusedMM.c:512-605);
+ * 0: every tuple follows the general pipeline (always accumulates).  Returns
+ * the previous setting. */
+int fusedMM_amd_set_opt(int enable);
+
+/* Tuning knobs of the heavy-row split: rows with more than `heavy_deg` edges
+ * are cut into segments of `seg_len` edges (0, 0 restores the K-dependent
+ * defaults).  For tests and experiments. */
+void fusedMM_amd_set_split(int64_t heavy_deg, int seg_len);
+
+/*
+ * Per-kernel timing with HIP events on the stream the kernels run on.
+ * enable != 0 starts a fresh recording (up to 512 calls are kept); the summary
+ * waits for the recorded events and returns the number of calls and the summed
+ * milliseconds of the row kernel, the segment kernel and the merge kernel.
+ */
+void fusedMM_amd_timing(int enable);
+int fusedMM_amd_timing_summary(double *rows_ms, double *segments_ms, double *merge_ms);
+
+/* Counters of the last call on this thread's device: heavy rows queued, edge
+ * segments queued, heavy rows that did not fit the queue.  Waits for the device. */
+int fusedMM_amd_last_split(unsigned int *heavy_rows, unsigned int *segments, unsigned int *overflow);
+
+/* Release every device buffer the library holds (work queues, staging). */
+void fusedMM_amd_finalize(void);
+
+#ifdef __cplusplus
+}
+#endif
+
+#endif /* FUSEDMM_AMD_H */

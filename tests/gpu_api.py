@@ -1,0 +1,70 @@
+"""Helpers for the GPU parity tests: run the C ABI on device or host operands
+and mirror the library's choice of wavefront layout so the oracle can be asked
+for the same summation order."""
+import numpy as np
+
+import fusedmm_amd as fa
+
+TKERN_MSG = {"g": fa.MSG_GCN, "m": fa.MSG_SPMM, "s": fa.MSG_SIGMOID, "t": fa.MSG_TDIST, "f": fa.MSG_FR}
+
+
+def layout_for(k, vec_ok=True):
+    """(V, L, S): floats per load, lanes per neighbour row, sub-waves per wave --
+    the rule in fusedmm_capi.hip:pick_shape."""
+    if vec_ok and k % 4 == 0:
+        if k <= 32:
+            L = 8
+        elif k <= 64:
+            L = 16
+        elif k <= 128:
+            L = 32
+        else:
+            L = 64
+        return 4, L, 64 // L
+    return 1, 64, 1
+
+
+def default_split(k):
+    """(heavy_deg, seg_len) defaults of the library for feature width k."""
+    seg = max(64, 262144 // (4 * k))
+    return 2 * seg, seg
+
+
+def run(imsg, g, X, Y, Z, beta=0.0, bits=32, where="device", m=None, k=None, ldx=None, ldy=None, ldz=None,
+        nnz=None):
+    """Call fusedMM_csr.  where='device': operands copied to the GPU with torch
+    and passed as device addresses; 'host': numpy arrays passed as they are.
+    Returns (status, Z as numpy)."""
+    m = g["rows"] if m is None else m
+    k = Y.shape[1] if k is None else k
+    ldx = (X.shape[1] if X is not None else k) if ldx is None else ldx
+    ldy = Y.shape[1] if ldy is None else ldy
+    ldz = Z.shape[1] if ldz is None else ldz
+    nnz = g["nnz"] if nnz is None else nnz
+    if where == "host":
+        Zh = np.ascontiguousarray(Z).copy()
+        rc = fa.fusedMM_csr(imsg, m, g["cols"], k, 1.0, nnz, g["rows"], g["cols"], g["val"], g["indx"],
+                            np.ascontiguousarray(g["pntrb"]), np.ascontiguousarray(g["pntre"]),
+                            X, ldx, Y, ldy, beta, Zh, ldz, index_bits=bits)
+        return rc, Zh
+    import torch
+    dev = torch.device("cuda:0")
+    t = lambda a: None if a is None else torch.from_numpy(np.ascontiguousarray(a)).to(dev)
+    val, indx, pb, pe = t(g["val"]), t(g["indx"]), t(g["pntrb"]), t(g["pntre"])
+    Xd, Yd, Zd = t(X), t(Y), t(Z)
+    rc = fa.fusedMM_csr(imsg, m, g["cols"], k, 1.0, nnz, g["rows"], g["cols"], val, indx, pb, pe,
+                        Xd, ldx, Yd, ldy, beta, Zd, ldz, index_bits=bits)
+    torch.cuda.synchronize()
+    return rc, Zd.cpu().numpy()
+
+
+def set_kind(kind, bits=32):
+    return fa.load(bits).fusedMM_amd_set_sop_kind(kind)
+
+
+def last_split(bits=32):
+    import ctypes as C
+    h, s, o = C.c_uint(), C.c_uint(), C.c_uint()
+    rc = fa.load(bits).fusedMM_amd_last_split(C.byref(h), C.byref(s), C.byref(o))
+    assert rc == 0
+    return h.value, s.value, o.value
