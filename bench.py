@@ -1,0 +1,212 @@
+#!/usr/bin/env python3
+"""Benchmark of the fused SDDMM+SpMM hot path (fusedMM_csr) on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c2]
+
+A step is one fusedMM_csr call over the whole synthetic graph, operands already
+resident in HBM.  Prints ONE JSON line.  The default workload is the one the
+headline metric is quoted on: the sigmoid graph-embedding op at K=128 on a
+symmetric Erdos-Renyi graph with 2^20 nodes and 2^24 edges, int32 indices.
+"""
+import argparse
+import ctypes as C
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+PEAK_HBM_GBPS = 8000.0
+
+WORKLOADS = {
+    # name: (description, op letter, K, sop kind)
+    "c1": ("fr K=32, ER n=16384 nnz=262144 (cache-resident plumbing case)", "f", 32, "fr"),
+    "c2": ("sigmoid K=128, ER n=2^20 nnz=2^24, int32", "s", 128, "sigmoid"),
+    "c3": ("spmm K=256, R-MAT scale 22 edge factor 16, symmetrised", "m", 256, None),
+    "c3g": ("gcn K=256, R-MAT scale 22 edge factor 16, symmetrised", "g", 256, None),
+    "c4": ("tdist K=64, R-MAT scale 24 edge factor 16, symmetrised", "t", 64, "tdist"),
+    "c5": ("sigmoid K=512, Zipf(1.8) degrees n=2^21 nnz~4e7, hubs to 1e6", "s", 512, "sigmoid"),
+}
+
+
+def make_workload(name, scale_down=0):
+    """Graph + embeddings of a benchmark configuration.  scale_down shrinks the
+    node count by 2^scale_down (used by the tests, never by the default bench)."""
+    from fusedmm_amd import synth
+    sd = scale_down
+    if name == "c1":
+        n = 16384 >> sd
+        g = synth.er_graph(n, 8 * n, 1)
+        X = synth.uniform_matrix(n, 32, -1.0, 1.0, 1)
+        return g, X, X
+    if name == "c2":
+        n = (1 << 20) >> sd
+        g = synth.er_graph(n, 8 * n, 2)
+        return g, synth.uniform_matrix(n, 128, -0.5, 0.5, 2, 1), synth.uniform_matrix(n, 128, -0.5, 0.5, 2, 2)
+    if name in ("c3", "c3g"):
+        g = synth.rmat_graph(22 - sd, 16, 3)
+        g["val"] = synth.edge_values(g["nnz"], 3)
+        return g, None, synth.normal_matrix(g["rows"], 256, 3)
+    if name == "c4":
+        g = synth.rmat_graph(24 - sd, 16, 4)
+        n = g["rows"]
+        return g, synth.uniform_matrix(n, 64, -1.0, 1.0, 4, 1), synth.uniform_matrix(n, 64, -1.0, 1.0, 4, 2)
+    if name == "c5":
+        n = (1 << 21) >> sd
+        g = synth.zipf_graph(n, 1.8, min(1000000, n // 2), 40000000 >> sd, 5)
+        return g, synth.uniform_matrix(n, 512, -0.5, 0.5, 5, 1), synth.uniform_matrix(n, 512, -0.5, 0.5, 5, 2)
+    raise SystemExit("unknown workload %s" % name)
+
+
+def cpu_baseline(name, g, X, Y, tkern, kind_id, k, budget_s=12.0):
+    """The CPU oracle's OpenMP port timed on this host's cores, on a bounded
+    sample of the same workload: the first rows of the graph (m < rows is part
+    of the API).  Checker-side code: used here only to report a baseline."""
+    sys.path.insert(0, os.path.join(ROOT, "tests"))
+    from oracle_api import Oracle
+    from fusedmm_amd import synth
+    orc = Oracle(fast=True)
+    threads = orc.max_threads()
+    rows = g["rows"]
+    m = min(rows, 1 << 18)
+    nnz_s = int(g["pntre"][m - 1]) - int(g["pntrb"][0])
+    Z = np.zeros((m, k), np.float32)
+    ot = "t" if tkern == "f" else tkern
+    orc.baseline(ot, g, X, Y, Z, 0.0, kind_id, threads, m=m)  # warm-up, untimed
+    t_all = []
+    t0 = time.time()
+    while (len(t_all) < 3 or time.time() - t0 < budget_s) and len(t_all) < 200:
+        t1 = time.time()
+        orc.baseline(ot, g, X, Y, Z, 0.0, kind_id, threads, m=m)
+        t_all.append(time.time() - t1)
+    t = float(np.mean(t_all))
+    flops = synth.algorithmic_flops(tkern, k, nnz_s)
+    return {"value": flops / t / 1e9, "unit": "GFLOP/s", "cores": threads, "kind": "port",
+            "sample": "first %d of %d rows of the same workload (%d edges), %d calls, mean %.4f s/call"
+                      % (m, rows, nnz_s, len(t_all), t),
+            "edges_per_s": nnz_s / t,
+            "alg_GBps": synth.algorithmic_bytes(tkern, m, k, nnz_s) / t / 1e9}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--workload", default="c2", choices=sorted(WORKLOADS))
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--no-check", action="store_true", help="skip the spot check against the oracle")
+    args = ap.parse_args()
+    if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
+        print("bench.py: this path is built and measured on ONE GPU; --gpus %d is not supported "
+              "(rows are independent, see DESIGN.md for how it would shard)" % args.gpus, file=sys.stderr)
+        sys.exit(2)
+
+    import torch
+    import fusedmm_amd as fa
+    from fusedmm_amd import synth
+
+    desc, tkern, k, kind = WORKLOADS[args.workload]
+    bits = 32
+    lib = fa.load(bits)
+    kind_id = {None: 0, "sigmoid": 1, "tdist": 2, "fr": 3}[kind]
+    lib.fusedMM_amd_set_sop_kind(kind_id)
+    imsg = {"s": fa.MSG_SIGMOID, "t": fa.MSG_TDIST, "f": fa.MSG_FR, "m": fa.MSG_SPMM, "g": fa.MSG_GCN}[tkern]
+
+    t_gen = time.time()
+    g, X, Y = make_workload(args.workload)
+    t_gen = time.time() - t_gen
+    m, n, nnz = g["rows"], g["cols"], g["nnz"]
+
+    dev = torch.device("cuda:0")
+    up = lambda a: None if a is None else torch.from_numpy(np.ascontiguousarray(a)).to(dev)
+    d_val, d_indx, d_pb, d_pe = up(g["val"]), up(g["indx"]), up(g["pntrb"]), up(g["pntre"])
+    d_X = up(X)
+    d_Y = d_X if Y is X else up(Y)
+    d_Z = torch.zeros((m, k), dtype=torch.float32, device=dev)
+    stream = torch.cuda.current_stream().cuda_stream
+
+    def step():
+        rc = fa.fusedMM_csr(imsg, m, n, k, 1.0, nnz, m, n, d_val, d_indx, d_pb, d_pe, d_X, k, d_Y, k, 0.0, d_Z, k,
+                            index_bits=bits, stream=stream)
+        if rc != 0:
+            raise SystemExit("fusedMM_csr returned %d" % rc)
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    lib.fusedMM_amd_timing(1)
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step()
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - t0
+    r_ms, s_ms, g_ms = C.c_double(), C.c_double(), C.c_double()
+    ncalls = lib.fusedMM_amd_timing_summary(C.byref(r_ms), C.byref(s_ms), C.byref(g_ms))
+    lib.fusedMM_amd_timing(0)
+    ms_per_step = wall / args.steps * 1e3
+
+    flops = synth.algorithmic_flops(tkern, k, nnz)
+    b_alg = synth.algorithmic_bytes(tkern, m, k, nnz, 4)
+    value = flops / (ms_per_step * 1e-3) / 1e9
+
+    kern_ms = {"rows_kernel": r_ms.value / max(1, ncalls), "segments_kernel": s_ms.value / max(1, ncalls),
+               "merge_kernel": g_ms.value / max(1, ncalls)}
+    # dominant kernel: the one the time goes to.  Its algorithmic bytes are the
+    # whole call's when no row is split (the other two kernels then find empty
+    # queues); with split rows the three kernels together move B_alg, so the
+    # roofline is quoted on their summed duration.
+    hs = (C.c_uint(), C.c_uint(), C.c_uint())
+    lib.fusedMM_amd_last_split(C.byref(hs[0]), C.byref(hs[1]), C.byref(hs[2]))
+    split = hs[1].value > 0
+    dom_ms = sum(kern_ms.values()) if split else kern_ms["rows_kernel"]
+    achieved = b_alg / (dom_ms * 1e-3) / 1e9 if dom_ms > 0 else 0.0
+    roofline = {"bound": "hbm", "achieved": achieved, "peak": PEAK_HBM_GBPS, "unit": "GB/s",
+                "frac": achieved / PEAK_HBM_GBPS, "traffic": None,
+                "kernel": "rows_kernel+segments_kernel+merge_kernel" if split else "rows_kernel",
+                "kernel_ms": dom_ms, "algorithmic_bytes": b_alg}
+
+    checked = None
+    if not args.no_check:
+        # spot check against the oracle (checker only): first rows, wavefront order, bit for bit
+        sys.path.insert(0, os.path.join(ROOT, "tests"))
+        from oracle_api import Oracle
+        from gpu_api import layout_for, default_split
+        mm = min(m, 4096)
+        light = int((np.diff(g["rowptr"][:mm + 1]).max())) <= default_split(k)[0]
+        Zs = np.zeros((mm, k), np.float32)
+        V, L, S = layout_for(k)
+        Oracle().opt("t" if tkern == "f" else tkern, g, X, Y, Zs, 0.0, kind_id, mode=2 if light else 1,
+                     V=V, L=L, S=S, m=mm)
+        got = d_Z[:mm].cpu().numpy()
+        if light:
+            checked = bool(np.array_equal(got.view(np.uint32), Zs.view(np.uint32)))
+        else:
+            checked = bool(np.allclose(got, Zs, rtol=1e-3, atol=1e-4))
+
+    out = {
+        "metric": "GFLOP/s + HBM GB/s (% of peak), sigmoid K=128, 1 MI355X vs CPU OpenMP",
+        "value": value, "unit": "GFLOP/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": ms_per_step, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "f32", "data": "synthetic",
+        "config": {"workload": "%s: %s" % (args.workload, desc), "op": tkern, "K": k, "rows": m, "nnz": nnz,
+                   "index_bits": bits, "beta": 0.0, "graph_gen_s": round(t_gen, 2)},
+        "edges_per_s": nnz / (ms_per_step * 1e-3),
+        "hbm_GBps_algorithmic": b_alg / (ms_per_step * 1e-3) / 1e9,
+        "pct_peak_hbm": 100.0 * b_alg / (ms_per_step * 1e-3) / 1e9 / PEAK_HBM_GBPS,
+        "kernel_ms": kern_ms,
+        "split": {"heavy_rows": hs[0].value, "segments": hs[1].value, "overflow": hs[2].value},
+        "spot_check_vs_oracle": checked,
+        "roofline": roofline,
+    }
+    if not args.no_cpu:
+        out["cpu_baseline"] = cpu_baseline(args.workload, g, X, Y, tkern, kind_id, k)
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()

@@ -26,9 +26,9 @@ def ragged(bits=32, seed=3, rows=97, cols=131, hub_deg=600):
         if r in (0, 5, rows - 1):
             lists.append(np.empty(0, np.int64))
         elif r == 2:
-            lists.append(np.array([4, 9, 9, 30], np.int64))
+            lists.append(np.array([4, 9, 9, 30], np.int64) % cols)
         elif r == 7:
-            lists.append(np.array([50, 3, 77, 12, 3], np.int64))
+            lists.append(np.array([50, 3, 77, 12, 3], np.int64) % cols)
         elif r == 11:
             lists.append(rng.integers(0, cols, hub_deg, dtype=np.int64))
         else:

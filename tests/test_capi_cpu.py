@@ -1,0 +1,72 @@
+"""Host-side checks of the C ABI that need no GPU: the libraries load, export
+every entry point the headers declare, and reject malformed op tuples with the
+reference's status codes before touching the device."""
+import os
+import re
+
+import numpy as np
+import pytest
+
+import fusedmm_amd as fa
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def declared_entry_points():
+    names = set()
+    for h in ("fusedMM.h", "fusedmm_amd.h"):
+        text = open(os.path.join(ROOT, "include", h)).read()
+        text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+        names |= set(re.findall(r"\b((?:fusedMM_|sgfusedMM_)\w+)\s*\(", text))
+    names.discard("fusedMM_amd_sop_fn")
+    return sorted(names)
+
+
+@pytest.mark.parametrize("bits", [32, 64])
+def test_library_exports_declared_symbols(bits):
+    lib = fa.load(bits)
+    names = declared_entry_points()
+    assert "fusedMM_csr" in names and "fusedMM_csr_stream" in names and len(names) >= 12
+    for n in names:
+        assert hasattr(lib, n), n
+    assert set(names) == set(fa.EXPORTS)
+    assert lib.fusedMM_amd_index_bytes() * 8 == bits
+
+
+def test_header_constants_match_python_mirror():
+    text = open(os.path.join(ROOT, "include", "fusedMM.h")).read()
+    for name in ("VOP_COPY_RHS", "VOP_SUBR", "ROP_DOT", "ROP_NORMR", "SOP_UDEF", "VSC_MUL", "AOP_ADD", "AOP_MIN"):
+        m = re.search(r"#define\s+%s\s+(0x[0-9A-Fa-f]+)" % name, text)
+        assert m and int(m.group(1), 16) == getattr(fa, name), name
+    assert fa.MSG_SIGMOID == 0x11F12 and fa.MSG_TDIST == 0x11F55 and fa.MSG_SPMM == 0x11102 and fa.MSG_GCN == 0x10002
+
+
+@pytest.mark.parametrize("bits", [32, 64])
+def test_bad_tuples_rejected_like_the_reference(bits):
+    """Order and codes of reference fusedMM.c:610-628; no operand is read."""
+    it = np.int32 if bits == 32 else np.int64
+    p = np.zeros(4, it)
+    f = np.zeros(16, np.float32)
+    call = lambda imsg: fa.fusedMM_csr(imsg, 2, 2, 4, 1.0, 0, 2, 2, f, p, p, p, f, 4, f, 4, 0.0, f, 4, index_bits=bits)
+    assert call(0x11100) == fa.VOP_FAIL              # VOP_NOOP is not accepted
+    assert call(0x11108) == fa.VOP_FAIL
+    assert call(0x11162) == fa.ROP_FAIL
+    assert call(0x11202) == fa.SOP_FAIL
+    assert call(0x13102) == fa.VSC_FAIL
+    assert call(0x41102) == fa.AOP_FAIL
+    assert call(0x1110F) == fa.UNDEFINED_USER_FUNCTION   # VOP_UDEF: no user function on the device
+    assert call(0x111F2) == fa.UNDEFINED_USER_FUNCTION
+    assert call(0x1F102) == fa.UNDEFINED_USER_FUNCTION
+    assert call(0xF1102) == fa.UNDEFINED_USER_FUNCTION
+    # first failing stage wins
+    assert call(0x43208) == fa.VOP_FAIL
+
+
+def test_sop_kind_selection():
+    lib = fa.load(32)
+    prev = lib.fusedMM_amd_set_sop_kind(fa.SOP_KIND_FR)
+    assert lib.fusedMM_amd_get_sop_kind() == fa.SOP_KIND_FR
+    assert lib.fusedMM_amd_set_sop_kind(99) == -2
+    assert lib.fusedMM_amd_get_sop_kind() == fa.SOP_KIND_FR
+    lib.fusedMM_amd_set_sop_kind(prev)
+    assert lib.fusedMM_amd_set_opt(1) in (0, 1)

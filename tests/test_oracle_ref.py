@@ -1,0 +1,52 @@
+"""Live cross-check of the CPU oracle against the real reference, compiled from
+/root/reference by `make -C oracle ref`.  Skipped where that build is absent."""
+import numpy as np
+import pytest
+
+import graphs
+from oracle_api import MSG, SOP_NAMES, Ref, ref_available
+
+pytestmark = pytest.mark.skipif(not ref_available(), reason="oracle/_ref not built (needs /root/reference)")
+KIND_OF = {"s": "sigmoid", "t": "tdist", "f": "fr", "m": "spmm", "g": "gcn"}
+
+
+def bits_equal(a, b):
+    return np.array_equal(a.view(np.uint32), b.view(np.uint32))
+
+
+def test_table_bits(oracle):
+    assert bits_equal(oracle.table(), Ref("sigmoid").table())
+
+
+@pytest.mark.parametrize("kind", ["sigmoid", "tdist", "fr", "ll", "fa"])
+def test_sop_bodies_bits(oracle, kind):
+    rng = np.random.default_rng(3)
+    v = rng.uniform(-6, 6, 100000).astype(np.float32)
+    edges = (np.arange(2049) * 10.0 / 2048 - 5.0).astype(np.float32)
+    v = np.concatenate([v, edges, np.nextafter(edges, np.float32(9)), np.nextafter(edges, np.float32(-9))])
+    v = v[v != np.float32(5.0)]       # the reference indexes one past its table there
+    if kind != "sigmoid":
+        v = np.abs(v) + np.float32(1e-4)
+    assert bits_equal(oracle.sop(SOP_NAMES[kind], v), Ref(kind).sop(v))
+
+
+@pytest.mark.parametrize("bits", [32, 64])
+@pytest.mark.parametrize("t", ["s", "t", "f", "m", "g"])
+@pytest.mark.parametrize("k", [8, 33, 128])
+def test_generic_path_bits(oracle, bits, t, k):
+    kind = KIND_OF[t]
+    r = Ref(kind, bits)
+    sk = SOP_NAMES.get(kind, 0)
+    for g in (graphs.ragged(bits), graphs.with_values(graphs.tiny_er(300, 2500, 4, bits))):
+        X = graphs.features(g["rows"], k, 1, -1, 1, 1)
+        Y = graphs.features(g["cols"], k, 1, -1, 1, 2)
+        Z0 = graphs.features(g["rows"], k, 1, -1, 1, 3)
+        A, B = Z0.copy(), Z0.copy()
+        r.test(t, g, X, Y, A)
+        assert oracle.generic(MSG[t], g, X, Y, B, sop_kind=sk) == 0
+        assert bits_equal(A, B)
+        # m < rows
+        A, B = Z0.copy(), Z0.copy()
+        r.test(t, g, X, Y, A, m=g["rows"] // 2)
+        oracle.generic(MSG[t], g, X, Y, B, sop_kind=sk, m=g["rows"] // 2)
+        assert bits_equal(A, B)
