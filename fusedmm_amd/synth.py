@@ -100,57 +100,31 @@ def rmat_graph(scale, edge_factor, seed, a=0.57, b=0.19, c=0.19, d=0.05, index_b
     return _csr_from_keys(n, keys, index_bits)
 
 
-def zipf_graph(n, exponent, cap, target_nnz, seed, index_bits=32):
-    """Power-law out-degrees: deg_i ~ Zipf(exponent) capped at `cap`, rescaled so
-    the total is about target_nnz; neighbours uniform without replacement,
-    sorted.  A few hub rows reach the cap, most rows have degree 1."""
+def zipf_graph(n, exponent, cap, target_nnz, seed, index_bits=32, n_hubs=4):
+    """Power-law out-degrees: deg_i ~ Zipf(exponent) capped at `cap`, the
+    mid-range rescaled so the total is about target_nnz; `n_hubs` rows are set
+    to the cap so the load-balance stress is always present.  Neighbours are
+    uniform, distinct within a row, never the row itself, sorted."""
     rng = _rng(seed)
+    cap = min(cap, n - 1)
     deg = np.minimum(rng.zipf(exponent, n).astype(np.int64), cap)
-    # make sure the stress the configuration asks for is present: a few hubs at the cap
-    hubs = rng.choice(n, 4, replace=False)
-    deg[hubs] = min(cap, n - 1)
+    hubs = np.sort(rng.choice(n, n_hubs, replace=False))
+    deg[hubs] = 0
     tot = int(deg.sum())
-    if tot > target_nnz:  # trim the mid-range, keep hubs and degree-1 rows
-        scale_f = (target_nnz - deg[hubs].sum()) / max(1, tot - deg[hubs].sum())
-        mask = np.ones(n, bool)
-        mask[hubs] = False
-        deg[mask] = np.maximum(1, (deg[mask] * scale_f).astype(np.int64))
-    deg = np.minimum(deg, n - 1)
-    rowptr = np.zeros(n + 1, np.int64)
-    np.cumsum(deg, out=rowptr[1:])
-    nnz = int(rowptr[-1])
-    indx = np.empty(nnz, np.int64)
-    big = np.nonzero(deg > 64)[0]
-    small_mask = deg <= 64
-    # small rows: draw with replacement, then repair duplicates / self-loops row by row
-    rows_rep = np.repeat(np.arange(n, dtype=np.int64)[small_mask], deg[small_mask])
-    draw = rng.integers(0, n, rows_rep.size, dtype=np.int64)
-    pos = np.concatenate([np.arange(rowptr[i], rowptr[i + 1]) for i in big]) if big.size else np.empty(0, np.int64)
-    small_pos = np.ones(nnz, bool)
-    small_pos[pos] = False
-    indx[small_pos] = draw
-    for i in big:
-        dsz = int(deg[i])
-        pick = rng.choice(n - 1, dsz, replace=False).astype(np.int64)
-        pick[pick >= i] += 1  # skip the diagonal
-        indx[rowptr[i]:rowptr[i + 1]] = pick
-    # sort inside rows and repair duplicates/self loops of the small rows
-    order = np.lexsort((indx, np.repeat(np.arange(n, dtype=np.int64), deg)))
-    indx = indx[order]
-    rowid = np.repeat(np.arange(n, dtype=np.int64), deg)
-    bad = (indx == rowid)
-    bad[1:] |= (indx[1:] == indx[:-1]) & (rowid[1:] == rowid[:-1])
-    # nudge offenders to a free neighbour id (rare: ~deg^2/n per row)
-    for p in np.nonzero(bad)[0]:
-        i = rowid[p]
-        lo, hi = rowptr[i], rowptr[i + 1]
-        row = set(indx[lo:hi].tolist())
-        cnd = int(indx[p])
-        while cnd in row or cnd == i:
-            cnd = (cnd + 1) % n
-        indx[p] = cnd
-        indx[lo:hi] = np.sort(indx[lo:hi])
-    return graph_from_rowptr(n, n, rowptr, indx, None, index_bits)
+    budget = max(n, target_nnz - n_hubs * cap)
+    if tot > budget:
+        deg = np.maximum(1, (deg * (budget / tot)).astype(np.int64))
+    deg[hubs] = 0
+    rows_rep = np.repeat(np.arange(n, dtype=np.int64), deg)
+    draw = rng.integers(0, n - 1, rows_rep.size, dtype=np.int64)
+    draw += draw >= rows_rep                       # skip the diagonal
+    parts = [np.unique(rows_rep * n + draw)]       # duplicates inside a row collapse
+    for h in hubs:
+        pick = rng.permutation(n - 1)[:cap].astype(np.int64)
+        pick += pick >= h
+        parts.append(h * n + np.sort(pick))
+    keys = np.sort(np.concatenate(parts))
+    return _csr_from_keys(n, keys, index_bits)
 
 
 def uniform_matrix(n, k, lo, hi, seed, stream=1):

@@ -68,3 +68,43 @@ def last_split(bits=32):
     rc = fa.load(bits).fusedMM_amd_last_split(C.byref(h), C.byref(s), C.byref(o))
     assert rc == 0
     return h.value, s.value, o.value
+
+
+def oracle_mirror(oracle, tkern, g, X, Y, Z0, beta, sop_kind, k, heavy_deg, seg_len, vec_ok=True, m=None):
+    """What the library computes, operation for operation: rows up to heavy_deg
+    edges in wavefront order; longer rows cut into seg_len-edge segments, each
+    reduced in wavefront order, the partials folded in segment order starting
+    from zero, then added to Z when beta != 0."""
+    m = g["rows"] if m is None else m
+    V, L, S = layout_for(k, vec_ok)
+    ot = "t" if tkern == "f" else tkern
+    Z = Z0.copy()
+    oracle.opt(ot, g, X, Y, Z, beta=beta, sop_kind=sop_kind, mode=2, V=V, L=L, S=S, m=m)
+    deg = (g["pntre"][:m].astype(np.int64) - g["pntrb"][:m].astype(np.int64))
+    heavy = np.nonzero(deg > heavy_deg)[0]
+    if heavy.size == 0:
+        return Z
+    pb, pe, owner = [], [], []
+    for r in heavy:
+        b, e = int(g["pntrb"][r]), int(g["pntre"][r])
+        for s0 in range(b, e, seg_len):
+            pb.append(s0)
+            pe.append(min(e, s0 + seg_len))
+            owner.append(r)
+    it = g["indx"].dtype
+    g2 = dict(g)
+    g2.update(rows=len(pb), pntrb=np.array(pb, it), pntre=np.array(pe, it))
+    X2 = None if X is None else np.ascontiguousarray(X[np.array(owner)])
+    P = np.zeros((len(pb), k), np.float32)
+    oracle.opt(ot, g2, X2, Y, P, beta=0.0, sop_kind=sop_kind, mode=2, V=V, L=L, S=S)
+    owner = np.array(owner)
+    for r in heavy:
+        a = np.zeros(k, np.float32)
+        for q in np.nonzero(owner == r)[0]:
+            a = (a + P[q]).astype(np.float32)
+        Z[r] = a if beta == 0.0 else (Z0[r] + a).astype(np.float32)
+    return Z
+
+
+def set_split(heavy_deg, seg_len, bits=32):
+    fa.load(bits).fusedMM_amd_set_split(heavy_deg, seg_len)

@@ -1,0 +1,177 @@
+"""General op tuples on the GPU, and the corners of the fusedMM_csr contract."""
+import os
+
+import numpy as np
+import pytest
+
+import checks
+import fusedmm_amd as fa
+import gpu_api
+import graphs
+from oracle_api import MSG, SOP_NAMES
+
+pytestmark = pytest.mark.gpu
+GOLD = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden")
+
+
+def test_tuple_sweep_against_reference_golden(oracle):
+    """168 op tuples: the reference's general pipeline (golden Z) vs the GPU's
+    runtime-switched kernel.  Sums differ in order only; max/min are exact."""
+    d = np.load(os.path.join(GOLD, "tuples_i32.npz"))
+    rows, cols = (int(v) for v in d["shape"])
+    g = {"rows": rows, "cols": cols, "nnz": int(d["indx"].size), "pntrb": d["pntrb"], "pntre": d["pntre"],
+         "indx": d["indx"], "val": d["val"]}
+    gpu_api.set_kind(SOP_NAMES["tdist"], 32)
+    lib = fa.load(32)
+    prev = lib.fusedMM_amd_set_opt(0)      # the golden Z comes from the general pipeline: always accumulates
+    try:
+        for imsg, want in zip(d["msgs"], d["Z"]):
+            imsg = int(imsg)
+            print("tuple", hex(imsg), flush=True)
+            rc, Z = gpu_api.run(imsg, g, d["X"], d["Y"], d["Z0"], bits=32)
+            assert rc == 0, hex(imsg)
+            checks.assert_close(Z, want, 3e-5, 1e-5 * float(np.abs(want).max()), None, hex(imsg))
+    finally:
+        lib.fusedMM_amd_set_opt(prev)
+
+
+@pytest.mark.parametrize("bits", [32, 64])
+def test_general_pipeline_always_accumulates(oracle, bits):
+    """opt off: the pattern tuples follow the general rule (beta ignored)."""
+    g = graphs.ragged(bits, hub_deg=50)
+    k = 32
+    Y = graphs.features(g["cols"], k, 4, -0.5, 0.5, 2)
+    Z0 = graphs.features(g["rows"], k, 4, -1, 1, 3)
+    lib = fa.load(bits)
+    prev = lib.fusedMM_amd_set_opt(0)
+    try:
+        rc, Z = gpu_api.run(MSG["m"], g, None, Y, Z0, beta=0.0, bits=bits)
+    finally:
+        lib.fusedMM_amd_set_opt(prev)
+    assert rc == 0
+    want = Z0.copy()
+    oracle.generic(MSG["m"], g, None, Y, want)
+    np.testing.assert_allclose(Z, want, rtol=1e-5, atol=1e-5)
+    assert np.abs(Z[0] - Z0[0]).max() == 0            # empty row untouched
+
+
+@pytest.mark.parametrize("where", ["device", "host"])
+def test_m_smaller_than_rows_and_split_pointers(oracle, where):
+    g = graphs.split_pointers(graphs.ragged(32, hub_deg=70))
+    k = 64
+    X = graphs.features(g["rows"], k, 5, -0.5, 0.5, 1)
+    Y = graphs.features(g["cols"], k, 5, -0.5, 0.5, 2)
+    Z0 = graphs.features(g["rows"], k, 5, -1, 1, 3)
+    gpu_api.set_kind(SOP_NAMES["sigmoid"], 32)
+    m = 41
+    rc, Z = gpu_api.run(MSG["s"], g, X, Y, Z0, beta=0.0, bits=32, where=where, m=m)
+    assert rc == 0
+    want = Z0.copy()
+    oracle.opt("s", g, X, Y, want, beta=0.0, sop_kind=1, mode=2, V=4, L=16, S=4, m=m)
+    np.testing.assert_array_equal(Z.view(np.uint32), want.view(np.uint32))
+    np.testing.assert_array_equal(Z[m:], Z0[m:])      # rows beyond m untouched
+
+
+@pytest.mark.parametrize("where", ["device", "host"])
+def test_leading_dimensions_larger_than_k(oracle, where):
+    g = graphs.ragged(32, hub_deg=70)
+    k, ldx, ldy, ldz = 48, 52, 64, 56
+    X = graphs.features(g["rows"], ldx, 6, -0.5, 0.5, 1)
+    Y = graphs.features(g["cols"], ldy, 6, -0.5, 0.5, 2)
+    Z0 = graphs.features(g["rows"], ldz, 6, -1, 1, 3)
+    gpu_api.set_kind(SOP_NAMES["tdist"], 32)
+    rc, Z = gpu_api.run(MSG["t"], g, X, Y, Z0, beta=1.0, bits=32, where=where, k=k)
+    assert rc == 0
+    want = Z0.copy()
+    oracle.opt("t", g, X, Y, want, beta=1.0, sop_kind=2, mode=2, V=4, L=16, S=4, k=k)
+    np.testing.assert_array_equal(Z.view(np.uint32), want.view(np.uint32))
+    np.testing.assert_array_equal(Z[:, k:], Z0[:, k:])   # padding columns untouched
+
+
+def test_unaligned_operands_take_the_scalar_layout(oracle):
+    """ldy not a multiple of 4: 16-byte gathers are impossible; the 4-byte layout is used."""
+    g = graphs.ragged(32, hub_deg=70)
+    k, ldy = 64, 65
+    X = graphs.features(g["rows"], k, 7, -0.5, 0.5, 1)
+    Y = graphs.features(g["cols"], ldy, 7, -0.5, 0.5, 2)
+    Z0 = np.zeros((g["rows"], k), np.float32)
+    gpu_api.set_kind(SOP_NAMES["sigmoid"], 32)
+    rc, Z = gpu_api.run(MSG["s"], g, X, Y, Z0, bits=32, k=k)
+    assert rc == 0
+    want = Z0.copy()
+    oracle.opt("s", g, X, Y, want, sop_kind=1, mode=2, V=1, L=64, S=1, k=k)
+    np.testing.assert_array_equal(Z.view(np.uint32), want.view(np.uint32))
+
+
+def test_x_and_y_are_the_same_buffer(oracle):
+    """Embedding training passes A = B (config 1 of the benchmark list)."""
+    import torch
+    g = graphs.tiny_er(300, 2400, 12)
+    k = 32
+    E = graphs.features(300, k, 8, -1, 1, 1)
+    dev = torch.device("cuda:0")
+    t = lambda a: torch.from_numpy(np.ascontiguousarray(a)).to(dev)
+    dE, Z = t(E), torch.zeros((300, k), device=dev)
+    val, indx, pb, pe = t(g["val"]), t(g["indx"]), t(g["pntrb"]), t(g["pntre"])
+    gpu_api.set_kind(SOP_NAMES["fr"], 32)
+    rc = fa.fusedMM_csr(fa.MSG_FR, 300, 300, k, 1.0, g["nnz"], 300, 300, val, indx, pb, pe, dE, k, dE, k, 0.0, Z, k)
+    assert rc == 0
+    torch.cuda.synchronize()
+    want = np.zeros((300, k), np.float32)
+    oracle.opt("t", g, E, E, want, sop_kind=3, mode=2, V=4, L=8, S=8)
+    np.testing.assert_array_equal(Z.cpu().numpy().view(np.uint32), want.view(np.uint32))
+    assert np.isfinite(want).all()                    # no self loops => no 1/0
+
+
+def test_empty_inputs():
+    k = 16
+    Y = graphs.features(5, k, 9)
+    Z0 = graphs.features(4, k, 9, stream=3)
+    empty = {"rows": 4, "cols": 5, "nnz": 0, "pntrb": np.zeros(4, np.int32), "pntre": np.zeros(4, np.int32),
+             "indx": np.zeros(1, np.int32), "val": np.zeros(1, np.float32)}
+    rc, Z = gpu_api.run(MSG["m"], empty, None, Y, Z0, beta=0.0)
+    assert rc == 0 and not Z.any()                    # beta == 0 overwrites even empty rows
+    rc, Z = gpu_api.run(MSG["m"], empty, None, Y, Z0, beta=1.0)
+    assert rc == 0 and np.array_equal(Z, Z0)
+    rc, Z = gpu_api.run(MSG["m"], empty, None, Y, Z0, beta=0.0, m=0)
+    assert rc == 0 and np.array_equal(Z, Z0)          # m == 0: nothing happens
+
+
+def test_k_beyond_supported_maximum_is_an_error():
+    g = graphs.tiny_er(20, 30, 2)
+    k = 2052
+    Y = np.zeros((20, k), np.float32)
+    rc, _ = gpu_api.run(MSG["g"], g, None, Y, np.zeros((20, k), np.float32))
+    assert rc == fa.FAIL
+
+
+@pytest.mark.parametrize("bits", [32, 64])
+def test_golden_ops_on_gpu(oracle, bits):
+    """The reference's own outputs (golden fixtures) within the stated tolerances."""
+    d = np.load(os.path.join(GOLD, "ops_i%d.npz" % bits))
+    it = np.int32 if bits == 32 else np.int64
+    for gname in ("ragged", "er"):
+        rows, cols = (int(v) for v in d[gname + "_shape"])
+        g = {"rows": rows, "cols": cols, "nnz": int(d[gname + "_indx"].size), "pntrb": d[gname + "_pntrb"].astype(it),
+             "pntre": d[gname + "_pntre"].astype(it), "indx": d[gname + "_indx"].astype(it), "val": d[gname + "_val"]}
+        deg = (g["pntre"] - g["pntrb"]).astype(np.int64)
+        for k in (16, 40):
+            X, Y = d["%s_X%d" % (gname, k)], d["%s_Y%d" % (gname, k)]
+            for t, kind in (("s", "sigmoid"), ("t", "tdist"), ("f", "fr"), ("m", None), ("g", None)):
+                sk = SOP_NAMES[kind] if kind else 0
+                gpu_api.set_kind(sk, bits)
+                rc, Z = gpu_api.run(MSG[t], g, X, Y, np.zeros((rows, k), np.float32), bits=bits)
+                assert rc == 0
+                want = d["%s_%s_k%d_fusedmm" % (gname, t, k)]
+                rtol, atol = (1e-5, 1e-6) if t in ("g", "m") else (1e-4, 1e-6)
+                es = np.zeros(int(g["pntre"].max()), np.float32)
+                tmp = np.zeros((rows, k), np.float32)
+                oracle.opt("t" if t == "f" else t, g, X, Y, tmp, sop_kind=sk, mode=1, edge_s=es if kind else None)
+                r_, slots = checks.edge_rows(g)
+                d_abs = np.ones(slots.size) if t == "g" else (np.abs(g["val"][slots]).astype(np.float64) if t == "m"
+                                                               else np.abs(oracle.sop(sk, es[slots])).astype(np.float64))
+                # the golden Z is itself a sequential fp32 sum over deg edges
+                extra = 2 * checks.EPS32 * np.maximum(deg, 1)[:, None] * checks.abs_term_sum(t, g, X, Y, d_abs)
+                if t == "s":
+                    extra = extra + checks.sigmoid_flip_slack(oracle.table(), g, X, Y)[0]
+                checks.assert_close(Z, want, rtol, atol, extra, "%s %s k=%d" % (gname, t, k))
