@@ -22,6 +22,12 @@ sys.path.insert(0, ROOT)
 
 PEAK_HBM_GBPS = 8000.0
 
+# HBM bytes per launch of the dominant kernel from rocprofv3 --pmc FETCH_SIZE and
+# WRITE_SIZE, each scaled by the same counter's reading for a plain 1 GiB copy
+# (profiles/rows_kernel_sigmoid_k128_c2.md).  Measured, not computed: refreshed
+# whenever the kernel changes.
+MEASURED_TRAFFIC_BYTES = {"c2": 10014758534}
+
 WORKLOADS = {
     # name: (description, op letter, K, sop kind)
     "c1": ("fr K=32, ER n=16384 nnz=262144 (cache-resident plumbing case)", "f", 32, "fr"),
@@ -100,6 +106,8 @@ def main():
     ap.add_argument("--workload", default="c2", choices=sorted(WORKLOADS))
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-check", action="store_true", help="skip the spot check against the oracle")
+    ap.add_argument("--copy-probe", action="store_true",
+                    help="also launch a plain 1 GiB copy kernel (yardstick for rocprofv3 --pmc FETCH_SIZE/WRITE_SIZE)")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py: this path is built and measured on ONE GPU; --gpus %d is not supported "
@@ -136,6 +144,14 @@ def main():
         if rc != 0:
             raise SystemExit("fusedMM_csr returned %d" % rc)
 
+    if args.copy_probe:
+        src = torch.ones(1 << 28, dtype=torch.float32, device=dev)
+        dst = torch.empty_like(src)
+        for _ in range(3):
+            assert lib.fusedMM_amd_copy_probe(dst.data_ptr(), src.data_ptr(), 1 << 30, stream) == 0
+        torch.cuda.synchronize()
+        del src, dst
+
     for _ in range(args.warmup):
         step()
     torch.cuda.synchronize()
@@ -166,7 +182,7 @@ def main():
     dom_ms = sum(kern_ms.values()) if split else kern_ms["rows_kernel"]
     achieved = b_alg / (dom_ms * 1e-3) / 1e9 if dom_ms > 0 else 0.0
     roofline = {"bound": "hbm", "achieved": achieved, "peak": PEAK_HBM_GBPS, "unit": "GB/s",
-                "frac": achieved / PEAK_HBM_GBPS, "traffic": None,
+                "frac": achieved / PEAK_HBM_GBPS, "traffic": MEASURED_TRAFFIC_BYTES.get(args.workload),
                 "kernel": "rows_kernel+segments_kernel+merge_kernel" if split else "rows_kernel",
                 "kernel_ms": dom_ms, "algorithmic_bytes": b_alg}
 

@@ -35,7 +35,8 @@ NOT_ENOUGH_MEM, UNDEFINED_USER_FUNCTION, NO_OPT_IMPL = -1, 64, 128
 EXPORTS = ("fusedMM_csr", "fusedMM_csr_stream", "sgfusedMM_csr", "fusedMM_amd_index_bytes",
            "fusedMM_amd_set_sop_kind", "fusedMM_amd_get_sop_kind", "fusedMM_amd_set_sop_callback",
            "fusedMM_amd_set_opt", "fusedMM_amd_set_split", "fusedMM_amd_timing",
-           "fusedMM_amd_timing_summary", "fusedMM_amd_last_split", "fusedMM_amd_finalize")
+           "fusedMM_amd_timing_summary", "fusedMM_amd_last_split", "fusedMM_amd_copy_probe",
+           "fusedMM_amd_finalize")
 
 _libs = {}
 
@@ -77,6 +78,8 @@ def load(index_bits=32):
     lib.fusedMM_amd_timing_summary.restype = C.c_int
     lib.fusedMM_amd_last_split.argtypes = [C.POINTER(C.c_uint)] * 3
     lib.fusedMM_amd_last_split.restype = C.c_int
+    lib.fusedMM_amd_copy_probe.argtypes = [vp, vp, C.c_int64, vp]
+    lib.fusedMM_amd_copy_probe.restype = C.c_int
     assert lib.fusedMM_amd_index_bytes() * 8 == index_bits
     _libs[index_bits] = lib
     return lib

@@ -630,6 +630,18 @@ int fusedMM_amd_last_split(unsigned int *heavy_rows, unsigned int *segments, uns
    return FUSEDMM_SUCCESS_RETURN;
 }
 
+int fusedMM_amd_copy_probe(void *dst, const void *src, int64_t bytes, void *stream)
+{
+   if (!dst || !src || bytes < 16 || (bytes & 15) || !aligned16(dst) || !aligned16(src)) return FUSEDMM_FAIL_RETURN;
+   std::lock_guard<std::mutex> lock(g.mu);
+   DeviceState *d = nullptr;
+   int st = device_state(&d);
+   if (st) return st;
+   hipLaunchKernelGGL(copy_probe_kernel, dim3((unsigned int)(d->num_cu * 8)), dim3(kBlockThreads), 0, (hipStream_t)stream,
+                      (float4 *)dst, (const float4 *)src, bytes / 16);
+   return hip_status(hipGetLastError(), "copy probe launch");
+}
+
 void fusedMM_amd_finalize(void)
 {
    std::lock_guard<std::mutex> lock(g.mu);

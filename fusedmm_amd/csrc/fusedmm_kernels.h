@@ -681,4 +681,12 @@ __global__ __launch_bounds__(kBlockThreads) void merge_kernel(const Params<IdxT>
    }
 }
 
+// Plain 16-byte copy of known size: the yardstick the HBM traffic counters
+// (FETCH_SIZE / WRITE_SIZE) of the kernels above are scaled by.
+__global__ __launch_bounds__(kBlockThreads) void copy_probe_kernel(float4 *dst, const float4 *src, int64_t n16)
+{
+   for (int64_t i = (int64_t)blockIdx.x * kBlockThreads + threadIdx.x; i < n16; i += (int64_t)gridDim.x * kBlockThreads)
+      dst[i] = src[i];
+}
+
 }  // namespace fmm

@@ -103,6 +103,12 @@ int fusedMM_amd_timing_summary(double *rows_ms, double *segments_ms, double *mer
  * segments queued, heavy rows that did not fit the queue.  Waits for the device. */
 int fusedMM_amd_last_split(unsigned int *heavy_rows, unsigned int *segments, unsigned int *overflow);
 
+/* Copy `bytes` (a multiple of 16, device memory, 16-byte aligned) with a plain
+ * grid-stride kernel on `stream`, asynchronously.  A measuring aid: hardware
+ * traffic counters of the kernels are scaled by what they read for this copy
+ * of known size. */
+int fusedMM_amd_copy_probe(void *dst, const void *src, int64_t bytes, void *stream);
+
 /* Release every device buffer the library holds (work queues, staging). */
 void fusedMM_amd_finalize(void);
 
