@@ -211,9 +211,11 @@ int launch_instance(const Params<idx_t> &p, const Launch &l)
    const int64_t need = (p.m + kWavesPerBlock - 1) / kWavesPerBlock;
    int64_t gr = (int64_t)l.num_cu * (l.blocks_per_cu > 0 ? l.blocks_per_cu : occ_rows);
    if (gr > need) gr = need;
+   Params<idx_t> pr = p;
+   pr.row_counters = (gr * kWavesPerBlock >= kRowCounters) ? kRowCounters : 1;
    const int64_t gs = (int64_t)l.num_cu * (l.blocks_per_cu > 0 ? l.blocks_per_cu : occ_segs);
    if (l.ev) FMM_HIP(hipEventRecord(l.ev[0], l.stream));
-   hipLaunchKernelGGL((rows_kernel<V, L, R, EXACT, OP, U, idx_t>), dim3((unsigned int)gr), dim3(kBlockThreads), 0, l.stream, p);
+   hipLaunchKernelGGL((rows_kernel<V, L, R, EXACT, OP, U, idx_t>), dim3((unsigned int)gr), dim3(kBlockThreads), 0, l.stream, pr);
    if (l.ev) FMM_HIP(hipEventRecord(l.ev[1], l.stream));
    hipLaunchKernelGGL((segments_kernel<V, L, R, EXACT, OP, U, idx_t>), dim3((unsigned int)gs), dim3(kBlockThreads), 0, l.stream, p);
    if (l.ev) FMM_HIP(hipEventRecord(l.ev[2], l.stream));
@@ -357,7 +359,7 @@ int run_on_device(const Args &a, const Plan &pl, int sop_kind, hipStream_t strea
    // not fit are processed whole by the row kernel, so this is never a
    // correctness question
    int64_t nnz_hint = (a.nnz > 0 && a.nnz < ((int64_t)1 << 40)) ? a.nnz : (int64_t)1 << 26;
-   int64_t cap_seg = nnz_hint / seg_len * 3 / 2 + 1024;
+   int64_t cap_seg = nnz_hint / seg_len * 3 / 2 + 1024;   // a row of d edges has at most d/seg_len + 1 segments
    int64_t cap_heavy = nnz_hint / heavy_deg + 1024;
    const int64_t max_partial_bytes = (int64_t)8 << 30;
    if (cap_seg * p.kpad * 4 > max_partial_bytes) cap_seg = max_partial_bytes / (p.kpad * 4);

@@ -46,7 +46,14 @@ struct Counters {
    unsigned int n_seg;      // edge segments queued
    unsigned int overflow;   // heavy rows that did not fit the queue (handled inline)
    unsigned int pad;
+   unsigned int pad2[28];         // keep the row counters on their own 128-byte lines
+   // Row claim counters.  Read-modify-writes on ONE address retire one per
+   // ~12 ns on this GPU however many CUs issue them; on distinct 128-byte
+   // lines they proceed in parallel.  So the row space is dealt to
+   // kRowCounters counters and a wave works its home counter first.
+   struct alignas(128) RowCounter { unsigned long long next; } rows[64];
 };
+constexpr int kRowCounters = 64;
 
 struct HeavyRow {
    int64_t row;
@@ -57,8 +64,11 @@ struct HeavyRow {
 struct SegDesc {
    int64_t row;
    unsigned int seg;       // segment number inside the row
-   unsigned int pad;
+   unsigned int len;       // edges per segment of this row
 };
+
+constexpr int kRowsPerClaim = 8;        // rows a wave claims at a time
+constexpr unsigned int kMaxSegsPerRow = 512;   // longer rows get longer segments
 
 template <typename IdxT>
 struct Params {
@@ -82,6 +92,7 @@ struct Params {
    float *partial;         // [cap_seg][kpad]
    unsigned int cap_heavy, cap_seg;
    int kpad;
+   int row_counters;       // claim counters in use: kRowCounters, or 1 when the grid has fewer waves
 };
 
 // ---- wave primitives --------------------------------------------------------
@@ -155,6 +166,19 @@ __device__ __forceinline__ int64_t wave_uniform<int64_t>(int64_t v)
 {
    int lo = __builtin_amdgcn_readfirstlane((int)(v & 0xFFFFFFFFll));
    int hi = __builtin_amdgcn_readfirstlane((int)(v >> 32));
+   return ((int64_t)hi << 32) | (uint32_t)lo;
+}
+
+// value held by lane `t` (wave-uniform t), delivered to every lane
+template <typename T>
+__device__ __forceinline__ T lane_value(T v, int t);
+template <>
+__device__ __forceinline__ int32_t lane_value<int32_t>(int32_t v, int t) { return __builtin_amdgcn_readlane(v, t); }
+template <>
+__device__ __forceinline__ int64_t lane_value<int64_t>(int64_t v, int t)
+{
+   int lo = __builtin_amdgcn_readlane((int)(v & 0xFFFFFFFFll), t);
+   int hi = __builtin_amdgcn_readlane((int)(v >> 32), t);
    return ((int64_t)hi << 32) | (uint32_t)lo;
 }
 
@@ -495,6 +519,34 @@ __device__ __forceinline__ const float *stage_table(const float *gtab, float *ld
    return lds;
 }
 
+// Turn the value an atomicAdd on counter `cur` returned (in lane 0) into a
+// chunk id, moving to another counter when this one is used up.  Returns -1
+// when every counter is used up; counters only grow, so every wave gets there.
+template <typename IdxT>
+__device__ __forceinline__ int64_t resolve_claim(const Params<IdxT> &p, unsigned long long claimed, int &cur, int nc,
+                                                 int64_t nchunks, int lane)
+{
+   for (;;)
+   {
+      const int64_t t = wave_uniform<int64_t>((int64_t)claimed);
+      const unsigned int mix = ((unsigned int)t * 2654435761u) >> 26;
+      const int64_t id = t * nc + (int64_t)((cur ^ mix) & (unsigned)(nc - 1));
+      if (id < nchunks) return id;
+      if (nc == 1) return -1;
+      // counter `cur` is spent (an id past the end can only occur in its last round)
+      unsigned long long seen = ~0ull;
+      if (lane < nc) seen = __hip_atomic_load(&p.ctr->rows[lane].next, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      const bool has = lane < nc && (int64_t)seen * nc < nchunks;
+      const unsigned long long mask = __ballot(has);
+      if (mask == 0) return -1;
+      const int sh = (cur + 1) & 63;
+      const unsigned long long rot = sh ? ((mask >> sh) | (mask << (64 - sh))) : mask;
+      cur = (sh + __builtin_ctzll(rot)) & 63;
+      claimed = 0;
+      if (lane == 0) claimed = atomicAdd(&p.ctr->rows[cur].next, 1ull);
+   }
+}
+
 // ---- kernel 1: one wavefront per row, heavy rows queued -------------------------
 template <int V, int L, int R, bool EXACT, int OP, int U, typename IdxT>
 __global__ __launch_bounds__(kBlockThreads) void rows_kernel(const Params<IdxT> p)
@@ -506,22 +558,48 @@ __global__ __launch_bounds__(kBlockThreads) void rows_kernel(const Params<IdxT> 
 
    const int lane = threadIdx.x & 63;
    const int sub = lane / L, sl = lane % L;
-   const int64_t wave0 = (int64_t)blockIdx.x * kWavesPerBlock + (threadIdx.x >> 6);
-   const int64_t nwaves = (int64_t)gridDim.x * kWavesPerBlock;
    const bool reads_x = op_reads_x<OP>(p.imessage);
    const int aop = p.imessage & 0xF0000;
    const bool generic = (OP == OP_GENERIC);
 
-   for (int64_t row = wave0; row < p.m; row += nwaves)
+   // Rows are claimed dynamically in chunks of kRowsPerClaim: degree-skewed
+   // graphs (R-MAT, power law) leave any static row -> wave map unbalanced.
+   // Counter c hands out, in round t, chunk  t * nc + ((c ^ mix(t)) & (nc-1)):
+   // every chunk has one owner, and a counter's chunks do not share row-id
+   // bits (R-MAT degrees depend on them).  A wave drains its home counter,
+   // then looks at all counters with one vector load and moves to the next one
+   // that still has chunks.  The next claim is issued before the current rows
+   // are walked, so its latency is hidden.
+   const int nc = p.row_counters;                        // 64, or 1 for tiny grids
+   const int64_t nchunks = (p.m + kRowsPerClaim - 1) / kRowsPerClaim;
+   int cur = (int)((blockIdx.x * kWavesPerBlock + (threadIdx.x >> 6)) & (unsigned)(nc - 1));
+   unsigned long long claimed = 0;
+   if (lane == 0) claimed = atomicAdd(&p.ctr->rows[cur].next, 1ull);
+   int64_t chunk = resolve_claim<IdxT>(p, claimed, cur, nc, nchunks, lane);
+   while (chunk >= 0)
    {
-      const IdxT jb = wave_uniform<IdxT>(p.pntrb[row]);
-      const IdxT je = wave_uniform<IdxT>(p.pntre[row]);
+   const int64_t row0 = chunk * kRowsPerClaim;
+   IdxT my_b = 0, my_e = 0;   // lane t holds the pointers of row0 + t
+   if (lane < kRowsPerClaim && row0 + lane < p.m)
+   {
+      my_b = p.pntrb[row0 + lane];
+      my_e = p.pntre[row0 + lane];
+   }
+   if (lane == 0) claimed = atomicAdd(&p.ctr->rows[cur].next, 1ull);
+   for (int t = 0; t < kRowsPerClaim && row0 + t < p.m; t++)
+   {
+      const int64_t row = row0 + t;
+      const IdxT jb = lane_value<IdxT>(my_b, t);
+      const IdxT je = lane_value<IdxT>(my_e, t);
       const int64_t deg = (int64_t)je - (int64_t)jb;
 
       if (deg > p.heavy_deg)
       {
          // queue the row for the segment kernel; if the queue is full, fall through
-         unsigned int nseg = (unsigned int)((deg + p.seg_len - 1) / p.seg_len);
+         // at most kMaxSegsPerRow partials per row: hub rows get longer segments
+         int64_t seg_len = p.seg_len;
+         if (deg > seg_len * (int64_t)kMaxSegsPerRow) seg_len = (deg + kMaxSegsPerRow - 1) / kMaxSegsPerRow;
+         unsigned int nseg = (unsigned int)((deg + seg_len - 1) / seg_len);
          unsigned int slot = 0, base = 0;
          if (lane == 0)
          {
@@ -534,7 +612,7 @@ __global__ __launch_bounds__(kBlockThreads) void rows_kernel(const Params<IdxT> 
          if (fits)
          {
             if (lane == 0) p.heavy[slot] = HeavyRow{row, base, nseg};
-            for (unsigned int s = lane; s < nseg; s += 64) p.segs[base + s] = SegDesc{row, s, 0u};
+            for (unsigned int s = lane; s < nseg; s += 64) p.segs[base + s] = SegDesc{row, s, (unsigned int)seg_len};
             continue;
          }
          // mark the slot unused (the merge kernel skips n_seg == 0) and do the row here
@@ -588,6 +666,8 @@ __global__ __launch_bounds__(kBlockThreads) void rows_kernel(const Params<IdxT> 
          store_slice<V, L, R, EXACT>(zrow, acc, sl, p.k);
       }
    }
+   chunk = resolve_claim<IdxT>(p, claimed, cur, nc, nchunks, lane);
+   }
 }
 
 // ---- kernel 2: one wavefront per queued edge segment -> partial Z -----------------
@@ -616,8 +696,9 @@ __global__ __launch_bounds__(kBlockThreads) void segments_kernel(const Params<Id
       if (row < 0) continue;   // slot of a row that was handled inline
       const IdxT rb = wave_uniform<IdxT>(p.pntrb[row]);
       const IdxT re = wave_uniform<IdxT>(p.pntre[row]);
-      const IdxT jb = rb + (IdxT)seg * (IdxT)p.seg_len;
-      IdxT je = jb + (IdxT)p.seg_len;
+      const IdxT seg_len = (IdxT)__builtin_amdgcn_readfirstlane((int)sd.len);
+      const IdxT jb = rb + (IdxT)seg * seg_len;
+      IdxT je = jb + seg_len;
       if (je > re) je = re;
 
       Slice<R> xs, acc;
@@ -638,45 +719,72 @@ __global__ __launch_bounds__(kBlockThreads) void segments_kernel(const Params<Id
    }
 }
 
-// ---- kernel 3: fold the partials of each heavy row, in segment order ----------------
-// One block per heavy row; thread t owns elements t, t+256, ...; the fold over
-// segments is sequential and therefore the same on every run.
+// ---- kernel 3: fold the partials of each heavy row -------------------------------------
+// One block per heavy row.  The block's 256 threads form G groups; group g folds
+// segments g, g+G, g+2G ... in ascending order starting from zero, then the G
+// group sums are added in ascending g.  G depends only on K, so the order of
+// every addition is fixed and results are the same on every run.
 template <typename IdxT>
 __global__ __launch_bounds__(kBlockThreads) void merge_kernel(const Params<IdxT> p, int generic)
 {
+   __shared__ float red[kBlockThreads];
    unsigned int nheavy = p.ctr->n_heavy;
    if (nheavy > p.cap_heavy) nheavy = p.cap_heavy;
    const int aop = p.imessage & 0xF0000;
+   const int cols = p.k < kBlockThreads ? p.k : kBlockThreads;   // elements handled per pass
+   int G = kBlockThreads / cols;                                  // groups (power of two not required)
+   if (G < 1) G = 1;
+   const int grp = threadIdx.x / cols, col = threadIdx.x % cols;
+   const bool active = grp < G;
    for (unsigned int h = blockIdx.x; h < nheavy; h += gridDim.x)
    {
       const HeavyRow hr = p.heavy[h];
       if (hr.n_seg == 0) continue;
       float *zrow = p.z + hr.row * p.ldz;
-      for (int e = threadIdx.x; e < p.k; e += kBlockThreads)
+      for (int e0 = 0; e0 < p.k; e0 += cols)
       {
+         const int e = e0 + col;
+         const bool live = active && e < p.k;
          const float *pp = p.partial + (int64_t)hr.seg_base * p.kpad + e;
-         float a;
-         if (generic) a = zrow[e];
-         else a = 0.0f;
-         if (generic && aop == kAopMax)
-            for (unsigned int s = 0; s < hr.n_seg; s++) a = fmaxf(a, pp[(int64_t)s * p.kpad]);
-         else if (generic && aop == kAopMin)
-            for (unsigned int s = 0; s < hr.n_seg; s++) a = fminf(a, pp[(int64_t)s * p.kpad]);
-         else
+         const bool is_max = generic && aop == kAopMax, is_min = generic && aop == kAopMin;
+         float a = is_max ? -__builtin_inff() : (is_min ? __builtin_inff() : 0.0f);
+         if (live)
          {
-            unsigned int s = 0;
-            for (; s + 8 <= hr.n_seg; s += 8)
+            unsigned int s = grp;
+            if (!is_max && !is_min)
             {
-               float v[8];
-#pragma unroll
-               for (int u = 0; u < 8; u++) v[u] = pp[(int64_t)(s + u) * p.kpad];
-#pragma unroll
-               for (int u = 0; u < 8; u++) a += v[u];
+               for (; s + 3u * G < hr.n_seg; s += 4u * G)
+               {
+                  const float v0 = pp[(int64_t)s * p.kpad], v1 = pp[(int64_t)(s + G) * p.kpad],
+                              v2 = pp[(int64_t)(s + 2u * G) * p.kpad], v3 = pp[(int64_t)(s + 3u * G) * p.kpad];
+                  a += v0; a += v1; a += v2; a += v3;
+               }
             }
-            for (; s < hr.n_seg; s++) a += pp[(int64_t)s * p.kpad];
+            for (; s < hr.n_seg; s += G)
+            {
+               const float v = pp[(int64_t)s * p.kpad];
+               a = is_max ? fmaxf(a, v) : (is_min ? fminf(a, v) : a + v);
+            }
          }
-         if (!generic && !p.beta_zero) a = zrow[e] + a;
-         zrow[e] = a;
+         __syncthreads();
+         red[threadIdx.x] = a;
+         __syncthreads();
+         if (live && grp == 0)
+         {
+            float t = red[col];
+            for (int g2 = 1; g2 < G; g2++)
+            {
+               const float v = red[g2 * cols + col];
+               t = is_max ? fmaxf(t, v) : (is_min ? fminf(t, v) : t + v);
+            }
+            if (generic)
+            {
+               const float zi = zrow[e];
+               t = is_max ? fmaxf(zi, t) : (is_min ? fminf(zi, t) : zi + t);
+            }
+            else if (!p.beta_zero) t = zrow[e] + t;
+            zrow[e] = t;
+         }
       }
    }
 }

@@ -24,6 +24,9 @@ def layout_for(k, vec_ok=True):
     return 1, 64, 1
 
 
+MAX_SEGS_PER_ROW = 512   # kMaxSegsPerRow of the kernels: longer rows get longer segments
+
+
 def default_split(k):
     """(heavy_deg, seg_len) defaults of the library for feature width k."""
     seg = max(64, 262144 // (4 * k))
@@ -72,9 +75,10 @@ def last_split(bits=32):
 
 def oracle_mirror(oracle, tkern, g, X, Y, Z0, beta, sop_kind, k, heavy_deg, seg_len, vec_ok=True, m=None):
     """What the library computes, operation for operation: rows up to heavy_deg
-    edges in wavefront order; longer rows cut into seg_len-edge segments, each
-    reduced in wavefront order, the partials folded in segment order starting
-    from zero, then added to Z when beta != 0."""
+    edges in wavefront order; longer rows cut into seg_len-edge segments (at
+    most MAX_SEGS_PER_ROW per row), each reduced in wavefront order; the merge
+    block's G thread groups fold segments g, g+G, ... in ascending order from
+    zero, the group sums are added in ascending g, then Z is added when beta != 0."""
     m = g["rows"] if m is None else m
     V, L, S = layout_for(k, vec_ok)
     ot = "t" if tkern == "f" else tkern
@@ -87,9 +91,10 @@ def oracle_mirror(oracle, tkern, g, X, Y, Z0, beta, sop_kind, k, heavy_deg, seg_
     pb, pe, owner = [], [], []
     for r in heavy:
         b, e = int(g["pntrb"][r]), int(g["pntre"][r])
-        for s0 in range(b, e, seg_len):
+        sl = seg_len if (e - b) <= seg_len * MAX_SEGS_PER_ROW else -(-(e - b) // MAX_SEGS_PER_ROW)
+        for s0 in range(b, e, sl):
             pb.append(s0)
-            pe.append(min(e, s0 + seg_len))
+            pe.append(min(e, s0 + sl))
             owner.append(r)
     it = g["indx"].dtype
     g2 = dict(g)
@@ -98,11 +103,16 @@ def oracle_mirror(oracle, tkern, g, X, Y, Z0, beta, sop_kind, k, heavy_deg, seg_
     P = np.zeros((len(pb), k), np.float32)
     oracle.opt(ot, g2, X2, Y, P, beta=0.0, sop_kind=sop_kind, mode=2, V=V, L=L, S=S)
     owner = np.array(owner)
+    G = max(1, 256 // min(k, 256))          # merge kernel: groups of a 256-thread block
     for r in heavy:
-        a = np.zeros(k, np.float32)
-        for q in np.nonzero(owner == r)[0]:
-            a = (a + P[q]).astype(np.float32)
-        Z[r] = a if beta == 0.0 else (Z0[r] + a).astype(np.float32)
+        mine = np.nonzero(owner == r)[0]
+        total = None
+        for grp in range(G):
+            a = np.zeros(k, np.float32)
+            for q in mine[grp::G]:
+                a = (a + P[q]).astype(np.float32)
+            total = a if total is None else (total + a).astype(np.float32)
+        Z[r] = total if beta == 0.0 else (Z0[r] + total).astype(np.float32)
     return Z
 
 

@@ -16,7 +16,7 @@ def with_values(g, seed=7):
     return g
 
 
-def ragged(bits=32, seed=3, rows=97, cols=131, hub_deg=600):
+def ragged(bits=32, seed=3, rows=97, cols=131, hub_deg=600, hub_rows=(11,)):
     """Rectangular, rows 0 and 5 and the last one empty, a duplicate column in
     row 2, one hub row much longer than the rest (with repeats), unsorted row 7."""
     rng = np.random.Generator(np.random.Philox(key=[seed, 0]))
@@ -29,7 +29,7 @@ def ragged(bits=32, seed=3, rows=97, cols=131, hub_deg=600):
             lists.append(np.array([4, 9, 9, 30], np.int64) % cols)
         elif r == 7:
             lists.append(np.array([50, 3, 77, 12, 3], np.int64) % cols)
-        elif r == 11:
+        elif r in hub_rows:
             lists.append(rng.integers(0, cols, hub_deg, dtype=np.int64))
         else:
             d = int(rng.integers(1, 24))

@@ -41,7 +41,7 @@ def test_split_rows_match_mirror(oracle, tkern, kind, k, bits, beta):
     h, s, o = gpu_api.last_split(bits)
     deg = g["pntre"] - g["pntrb"]
     assert h == int((deg > heavy_deg).sum()) and o == 0
-    assert s == int(np.ceil(deg[deg > heavy_deg] / seg_len).sum())
+    assert s == int(np.ceil(deg[deg > heavy_deg] / seg_len).sum())       # no row here exceeds 512 segments
     want = gpu_api.oracle_mirror(oracle, tkern, g, X, Y, Z0, beta, sk, k, heavy_deg, seg_len, vec_ok=(k % 4 == 0))
     np.testing.assert_array_equal(Z.view(np.uint32), want.view(np.uint32))
     rc, Z2 = gpu_api.run(MSG[tkern], g, X, Y, Z0, beta=beta, bits=bits)
@@ -75,7 +75,7 @@ def test_default_thresholds_hub_row(oracle, tkern, kind):
     assert rc == 0
     heavy_deg, seg_len = gpu_api.default_split(k)
     h, s, o = gpu_api.last_split(bits)
-    assert (h, s, o) == (1, -(-40000 // seg_len), 0)
+    assert (h, s, o) == (1, -(-40000 // seg_len), 0)                   # 79 segments of 512 edges
     want = gpu_api.oracle_mirror(oracle, tkern, g, X, Y, Z0, 0.0, sk, k, heavy_deg, seg_len)
     np.testing.assert_array_equal(Z.view(np.uint32), want.view(np.uint32))
 
@@ -84,10 +84,10 @@ def test_queue_overflow_is_handled_inline(oracle):
     """A caller-supplied nnz that is far too small undersizes the segment queue:
     rows that do not fit are processed whole by the row kernel; the answer stays right."""
     bits, k = 32, 64
-    g = graphs.ragged(bits, rows=40, cols=3000, hub_deg=9000)
+    g = graphs.ragged(bits, rows=40, cols=3000, hub_deg=2000, hub_rows=(11, 13, 17))
     Y = graphs.features(g["cols"], k, 3, -0.5, 0.5, 2)
     Z0 = np.zeros((g["rows"], k), np.float32)
-    gpu_api.set_split(8, 4, bits)              # 9000/4 = 2250 segments for the hub alone
+    gpu_api.set_split(8, 4, bits)              # 3 hubs x 500 segments + the short rows > 1024
     rc, Z = gpu_api.run(MSG["m"], g, None, Y, Z0, bits=bits, nnz=1)   # queue capacity falls to its floor (1024)
     assert rc == 0
     h, s, o = gpu_api.last_split(bits)
@@ -99,3 +99,20 @@ def test_queue_overflow_is_handled_inline(oracle):
     extra = 4 * checks.EPS32 * np.sqrt(np.maximum(deg, 1))[:, None] * \
         checks.abs_term_sum("m", g, None, Y, np.abs(g["val"][slots]).astype(np.float64))
     checks.assert_close(Z, Z64, 1e-5, 1e-6, extra, "overflow")
+
+
+def test_very_long_row_gets_longer_segments(oracle):
+    """A row that would need more than 512 segments is cut into 512-at-most longer ones."""
+    bits, k = 32, 64
+    g = graphs.ragged(bits, rows=30, cols=4000, hub_deg=40000)
+    Y = graphs.features(g["cols"], k, 2, -0.5, 0.5, 2)
+    Z0 = graphs.features(g["rows"], k, 2, -1, 1, 3)
+    gpu_api.set_split(16, 8, bits)
+    rc, Z = gpu_api.run(MSG["m"], g, None, Y, Z0, beta=1.0, bits=bits)
+    assert rc == 0
+    deg = (g["pntre"] - g["pntrb"]).astype(np.int64)
+    others = deg[(deg > 16) & (deg < 40000)]
+    h, s, o = gpu_api.last_split(bits)
+    assert o == 0 and s == int(np.ceil(others / 8).sum()) + -(-40000 // -(-40000 // 512))
+    want = gpu_api.oracle_mirror(oracle, "m", g, None, Y, Z0, 1.0, 0, k, 16, 8)
+    np.testing.assert_array_equal(Z.view(np.uint32), want.view(np.uint32))
