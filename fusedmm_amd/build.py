@@ -41,9 +41,40 @@ def build_one(index_bits, verbose=False):
     return out
 
 
+def timer_path(index_bits):
+    return os.path.join(HERE, "bin", "xfusedMMtime_i%d" % index_bits)
+
+
+def harness_lib_path(index_bits):
+    return os.path.join(HERE, "libfusedmm_harness_i%d.so" % index_bits)
+
+
+def _run(cmd, verbose):
+    if verbose:
+        print(" ".join(cmd), flush=True)
+    r = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
+    if r.returncode != 0:
+        sys.stderr.write(r.stdout)
+        raise RuntimeError("build step failed: " + " ".join(cmd))
+
+
+def build_timer(index_bits, verbose=False):
+    """The tester/timer executable (csrc/fusedMMtime.cpp) and the loader's C doorway."""
+    os.makedirs(os.path.join(HERE, "bin"), exist_ok=True)
+    exe = timer_path(index_bits)
+    _run([HIPCC, "-O2", "-std=c++17", "-fopenmp", "-DINDEXTYPE=int%d_t" % index_bits,
+          os.path.join(CSRC, "fusedMMtime.cpp"), "-o", exe, "-L" + HERE, "-lfusedmm_amd_i%d" % index_bits,
+          "-Wl,-rpath,$ORIGIN/..", "-L/opt/rocm/lib", "-lrocprofiler-sdk-roctx", "-Wl,-rpath,/opt/rocm/lib"], verbose)
+    _run(["g++", "-O2", "-std=c++17", "-fPIC", "-shared", "-DINDEXTYPE=int%d_t" % index_bits,
+          os.path.join(CSRC, "harness_capi.cpp"), "-o", harness_lib_path(index_bits)], verbose)
+    return exe
+
+
 def build_all(verbose=False):
     with ThreadPoolExecutor(2) as ex:
-        return list(ex.map(lambda b: build_one(b, verbose), (32, 64)))
+        libs = list(ex.map(lambda b: build_one(b, verbose), (32, 64)))
+        exes = list(ex.map(lambda b: build_timer(b, verbose), (32, 64)))
+    return libs + exes
 
 
 if __name__ == "__main__":

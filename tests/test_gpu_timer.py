@@ -1,0 +1,43 @@
+"""The tester/timer executable on a small .mtx: the reference's own workflow
+(`x...time -input f.mtx -T 1 -K k`) must pass its tester and print the CSV."""
+import os
+import subprocess
+
+import pytest
+
+from fusedmm_amd import build as fbuild
+from fusedmm_amd import synth
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.mark.parametrize("bits", [32, 64])
+@pytest.mark.parametrize("tkern,k", [("f", 32), ("s", 128), ("t", 64), ("m", 256), ("g", 40)])
+def test_timer_passes_its_tester(tmp_path, tkern, k, bits):
+    g = synth.er_graph(4096, 32768, 1, bits)
+    path = str(tmp_path / "er.mtx")
+    synth.write_mtx_symmetric(path, g)
+    exe = fbuild.timer_path(bits)
+    assert os.path.exists(exe)
+    r = subprocess.run([exe, "-input", path, "-T", "1", "-K", str(k), "-t", tkern, "-nrep", "3"],
+                       stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True, timeout=110)
+    print(r.stdout)
+    assert r.returncode == 0, r.stdout
+    assert "PASSED TEST" in r.stdout
+    lines = [l for l in r.stdout.splitlines() if "," in l]
+    assert lines[-2].startswith("Filename,NNZ,M,N,K,Trusted_exe_time,Test_exe_time,Speedup_exe_time")
+    f = lines[-1].split(",")
+    assert f[1:5] == [str(g["nnz"]), "4096", "4096", str(k)]
+    assert float(f[6]) > 0 and float(f[8]) > 0
+
+
+def test_timer_host_pointer_mode(tmp_path):
+    g = synth.er_graph(2048, 16384, 2, 64)
+    path = str(tmp_path / "er.mtx")
+    synth.write_mtx_symmetric(path, g)
+    r = subprocess.run([fbuild.timer_path(64), "-input", path, "-T", "1", "-K", "64", "-t", "s", "-nrep", "2",
+                        "-gpu", "0", "-skHd", "1", "-M", "1000"],
+                       stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True, timeout=110)
+    assert r.returncode == 0 and "PASSED TEST" in r.stdout, r.stdout
+    assert "Filename" not in r.stdout
+    assert r.stdout.strip().splitlines()[-1].split(",")[2] == "1000"
