@@ -45,6 +45,10 @@ def timer_path(index_bits):
     return os.path.join(HERE, "bin", "xfusedMMtime_i%d" % index_bits)
 
 
+def dropin_path(index_bits):
+    return os.path.join(HERE, "bin", "xdropin_example_i%d" % index_bits)
+
+
 def harness_lib_path(index_bits):
     return os.path.join(HERE, "libfusedmm_harness_i%d.so" % index_bits)
 
@@ -67,6 +71,10 @@ def build_timer(index_bits, verbose=False):
           "-Wl,-rpath,$ORIGIN/..", "-L/opt/rocm/lib", "-lrocprofiler-sdk-roctx", "-Wl,-rpath,/opt/rocm/lib"], verbose)
     _run(["g++", "-O2", "-std=c++17", "-fPIC", "-shared", "-DINDEXTYPE=int%d_t" % index_bits,
           os.path.join(CSRC, "harness_capi.cpp"), "-o", harness_lib_path(index_bits)], verbose)
+    # a reference-style caller in plain C (gcc, host pointers, its own SOP_UDEF_FUNC)
+    _run(["gcc", "-O2", "-DINDEXTYPE=int%d_t" % index_bits, "-DVALUETYPE=float",
+          os.path.join(CSRC, "dropin_example.c"), "-rdynamic", "-o", dropin_path(index_bits), "-L" + HERE,
+          "-lfusedmm_amd_i%d" % index_bits, "-Wl,-rpath,$ORIGIN/..", "-Wl,-rpath-link,/opt/rocm/lib", "-lm"], verbose)
     return exe
 
 

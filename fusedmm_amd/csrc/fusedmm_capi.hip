@@ -13,6 +13,7 @@
 #include <string.h>
 
 #include <mutex>
+#include <thread>
 #include <vector>
 
 #ifndef INDEXTYPE
@@ -417,12 +418,10 @@ bool is_device_pointer(const void *p)
    return attr.type == hipMemoryTypeDevice || attr.type == hipMemoryTypeManaged;
 }
 
-// Host-pointer mode: stage operands to the GPU, run, copy Z back.  Only the
-// first k columns of each Z row are written back, as the reference touches
-// nothing else.
-int run_staged(const Args &h, const Plan &pl, int sop_kind)
+// Host-pointer mode: copy the operands to the GPU.  On return `a` holds device
+// addresses and `slots` is one past the last edge slot any processed row uses.
+int stage_up(const Args &h, const Plan &pl, Args *a, int64_t *slots_out)
 {
-   if (h.m <= 0 || h.k < 1) return FUSEDMM_SUCCESS_RETURN;
    if (h.n <= 0) { FMM_LOG("n (rows of Y) must be positive for host operands"); return FUSEDMM_FAIL_RETURN; }
    DeviceState *d = nullptr;
    int st = device_state(&d);
@@ -457,21 +456,134 @@ int run_staged(const Args &h, const Plan &pl, int sop_kind)
    if (!overwrite)
       FMM_HIP(hipMemcpy2DAsync(d->stage[6].ptr, (size_t)h.ldz * 4, h.z, (size_t)h.ldz * 4, (size_t)h.k * 4, (size_t)h.m,
                                hipMemcpyHostToDevice, s));
-   Args a = h;
-   a.pntrb = (const idx_t *)d->stage[0].ptr;
-   a.pntre = (const idx_t *)d->stage[1].ptr;
-   a.indx = (const idx_t *)d->stage[2].ptr;
-   a.val = need_val ? (const float *)d->stage[3].ptr : nullptr;
-   a.x = pl.reads_x ? (const float *)d->stage[4].ptr : nullptr;
-   a.y = (const float *)d->stage[5].ptr;
-   a.z = (float *)d->stage[6].ptr;
-   if (a.nnz <= 0 || a.nnz > slots) a.nnz = slots;
-   st = run_on_device(a, pl, sop_kind, s);
-   if (st) return st;
-   FMM_HIP(hipMemcpy2DAsync(h.z, (size_t)h.ldz * 4, d->stage[6].ptr, (size_t)h.ldz * 4, (size_t)h.k * 4, (size_t)h.m,
-                            hipMemcpyDeviceToHost, s));
-   FMM_HIP(hipStreamSynchronize(s));
+   *a = h;
+   a->pntrb = (const idx_t *)d->stage[0].ptr;
+   a->pntre = (const idx_t *)d->stage[1].ptr;
+   a->indx = (const idx_t *)d->stage[2].ptr;
+   a->val = need_val ? (const float *)d->stage[3].ptr : nullptr;
+   a->x = pl.reads_x ? (const float *)d->stage[4].ptr : nullptr;
+   a->y = (const float *)d->stage[5].ptr;
+   a->z = (float *)d->stage[6].ptr;
+   if (a->nnz <= 0 || a->nnz > slots) a->nnz = slots;
+   *slots_out = slots;
    return FUSEDMM_SUCCESS_RETURN;
+}
+
+// Only the first k columns of each Z row are written back, as the reference
+// touches nothing else.
+int stage_down(const Args &h, const Args &a)
+{
+   FMM_HIP(hipMemcpy2DAsync(h.z, (size_t)h.ldz * 4, a.z, (size_t)h.ldz * 4, (size_t)h.k * 4, (size_t)h.m,
+                            hipMemcpyDeviceToHost, 0));
+   FMM_HIP(hipStreamSynchronize(0));
+   return FUSEDMM_SUCCESS_RETURN;
+}
+
+int run_staged(const Args &h, const Plan &pl, int sop_kind)
+{
+   if (h.m <= 0 || h.k < 1) return FUSEDMM_SUCCESS_RETURN;
+   Args a;
+   int64_t slots = 0;
+   int st = stage_up(h, pl, &a, &slots);
+   if (st) return st;
+   st = run_on_device(a, pl, sop_kind, 0);
+   if (st) return st;
+   return stage_down(h, a);
+}
+
+// ---- SOP_UDEF evaluated by the caller's host function ---------------------------------------
+// The reference calls SOP_UDEF_FUNC once per edge from inside its kernels
+// (genkern.base:487, 554; fusedMM.c:729).  Here: pass 1 on the GPU writes the
+// ROP result of every edge, the host applies the function to each of them,
+// pass 2 on the GPU runs the rest of the pipeline (MOP, AOP) with those
+// scalars as edge values.  Synchronous; device operands `a`, host copies of
+// the row pointers in h_pb / h_pe.
+template <int V, int L, int R, bool EXACT, int U>
+int launch_edge_scalar(const Params<idx_t> &p, float *s_out, int num_cu)
+{
+   int64_t blocks = (p.m + kWavesPerBlock - 1) / kWavesPerBlock;
+   if (blocks > (int64_t)num_cu * 8) blocks = (int64_t)num_cu * 8;
+   hipLaunchKernelGGL((edge_scalar_kernel<V, L, R, EXACT, U, idx_t>), dim3((unsigned int)blocks), dim3(kBlockThreads), 0, 0,
+                      p, s_out);
+   return hip_status(hipGetLastError(), "edge scalar launch");
+}
+
+int run_host_sop(const Args &a, const idx_t *h_pb, const idx_t *h_pe, int64_t slots, const Plan &pl,
+                 fusedMM_amd_sop_fn fn)
+{
+   if (a.m <= 0 || a.k < 1) return FUSEDMM_SUCCESS_RETURN;
+   if (a.k > kMaxK) { FMM_LOG("feature dimension k=%lld is beyond the supported maximum %d", (long long)a.k, kMaxK); return FUSEDMM_FAIL_RETURN; }
+   DeviceState *d = nullptr;
+   int st = device_state(&d);
+   if (st) return st;
+   const int vsc = GET_VSC_FLAG(a.imessage);
+   const bool overwrite = pl.opt_rule && a.beta == 0.0f;
+   if (overwrite)
+      FMM_HIP(hipMemset2DAsync(a.z, (size_t)a.ldz * 4, 0, (size_t)a.k * 4, (size_t)a.m, 0));
+   if (slots <= 0) return hip_status(hipStreamSynchronize(0), "hipStreamSynchronize");
+   st = grow(d->stage[7], (size_t)slots * sizeof(float));
+   if (st) return st;
+   float *d_s = (float *)d->stage[7].ptr;
+
+   // pass 1
+   const bool vec_ok = (a.k % 4 == 0) && (a.ldy % 4 == 0) && aligned16(a.y) && (a.ldx % 4 == 0) && aligned16(a.x);
+   Shape sh;
+   st = pick_shape((int)a.k, vec_ok, &sh);
+   if (st) return st;
+   Params<idx_t> p;
+   memset(&p, 0, sizeof(p));
+   p.pntrb = a.pntrb; p.pntre = a.pntre; p.indx = a.indx; p.val = a.val;
+   p.x = a.x ? a.x : a.y;   // tuples that never read X still index it; any valid row will do
+   p.y = a.y; p.m = a.m; p.ldx = a.x ? a.ldx : 0; p.ldy = a.ldy; p.k = (int)a.k; p.imessage = a.imessage;
+#define FMM_CASE(V_, L_, R_, X_, U_) \
+   if (sh.V == V_ && sh.L == L_ && sh.R == R_ && sh.exact == X_) st = launch_edge_scalar<V_, L_, R_, (X_ != 0), U_>(p, d_s, d->num_cu); else
+   FMM_CASE(4, 8, 1, 1, 8) FMM_CASE(4, 16, 1, 1, 8) FMM_CASE(4, 32, 1, 1, 8) FMM_CASE(4, 64, 1, 1, 8)
+   FMM_CASE(4, 64, 2, 1, 4) FMM_CASE(4, 8, 1, 0, 8) FMM_CASE(4, 16, 1, 0, 8) FMM_CASE(4, 32, 1, 0, 8)
+   FMM_CASE(4, 64, 1, 0, 8) FMM_CASE(4, 64, 2, 0, 4) FMM_CASE(4, 64, 4, 0, 2) FMM_CASE(4, 64, 8, 0, 1)
+   FMM_CASE(1, 64, 1, 0, 8) FMM_CASE(1, 64, 2, 0, 4) FMM_CASE(1, 64, 4, 0, 2) FMM_CASE(1, 64, 8, 0, 1)
+   st = FUSEDMM_FAIL_RETURN;
+#undef FMM_CASE
+   if (st) return st;
+   std::vector<float> hs((size_t)slots);
+   FMM_HIP(hipMemcpyAsync(hs.data(), d_s, (size_t)slots * sizeof(float), hipMemcpyDeviceToHost, 0));
+   FMM_HIP(hipStreamSynchronize(0));
+
+   // host SOP, rows dealt to a few threads (the function must be thread-safe, reference fusedMM.h:125-126)
+   unsigned int nthreads = std::thread::hardware_concurrency();
+   if (nthreads < 1) nthreads = 1;
+   if (nthreads > 16) nthreads = 16;
+   if ((int64_t)nthreads > a.m) nthreads = (unsigned int)a.m;
+   std::vector<std::thread> pool;
+   for (unsigned int t = 0; t < nthreads; t++)
+      pool.emplace_back([&, t]() {
+         const int64_t lo = a.m * t / nthreads, hi = a.m * (t + 1) / nthreads;
+         for (int64_t i = lo; i < hi; i++)
+            for (int64_t j = (int64_t)h_pb[i]; j < (int64_t)h_pe[i]; j++)
+            {
+               float out = hs[(size_t)j];
+               (void)fn(hs[(size_t)j], &out);
+               hs[(size_t)j] = out;
+            }
+      });
+   for (auto &th : pool) th.join();
+   FMM_HIP(hipMemcpyAsync(d_s, hs.data(), (size_t)slots * sizeof(float), hipMemcpyHostToDevice, 0));
+
+   // pass 2: same VOP / MOP / AOP, the scalar comes in as the edge value
+   Args a2 = a;
+   a2.val = d_s;
+   a2.imessage = GET_VOP_FLAG(a.imessage) | ROP_NOOP | SOP_COPY | vsc | GET_AOP_FLAG(a.imessage);
+   Plan p2;
+   st = make_plan(a2.imessage, 0, &p2);   // general rule: accumulate (Z was cleared above when it must be overwritten)
+   if (st) return st;
+   st = run_on_device(a2, p2, FUSEDMM_SOP_KIND_IDENTITY, 0);
+   if (st) return st;
+   return hip_status(hipStreamSynchronize(0), "hipStreamSynchronize");
+}
+
+fusedMM_amd_sop_fn host_sop_function()
+{
+   if (g.sop_fn) return g.sop_fn;
+   return (fusedMM_amd_sop_fn)dlsym(RTLD_DEFAULT, "SOP_UDEF_FUNC");
 }
 
 int entry(const Args &a, bool async, hipStream_t stream)
@@ -484,9 +596,40 @@ int entry(const Args &a, bool async, hipStream_t stream)
    int sop_kind = g.sop_kind;
    if (pl.needs_sop && sop_kind == FUSEDMM_SOP_KIND_HOST)
    {
-      FMM_LOG("SOP_UDEF with kind 'host' is not available in this build of the path; "
-              "select a device body with fusedMM_amd_set_sop_kind() or FUSEDMM_SOP_KIND");
-      return FUSEDMM_UNDEFINED_USER_FUNCTION;
+      if (GET_VSC_FLAG(a.imessage) == VSC_NOOP)
+         sop_kind = FUSEDMM_SOP_KIND_IDENTITY;   // the SOP result is never used
+      else
+      {
+         fusedMM_amd_sop_fn fn = host_sop_function();
+         if (!fn)
+         {
+            FMM_LOG("SOP_UDEF: no host SOP_UDEF_FUNC found and no device body selected "
+                    "(fusedMM_amd_set_sop_kind / FUSEDMM_SOP_KIND)");
+            return FUSEDMM_UNDEFINED_USER_FUNCTION;
+         }
+         if (async)
+         {
+            FMM_LOG("SOP_UDEF through a host function needs the synchronous entry point");
+            return FUSEDMM_UNDEFINED_USER_FUNCTION;
+         }
+         if (a.m <= 0 || a.k < 1) return FUSEDMM_SUCCESS_RETURN;
+         if (is_device_pointer(a.z))
+         {
+            std::vector<idx_t> hb((size_t)a.m), he((size_t)a.m);
+            FMM_HIP(hipMemcpy(hb.data(), a.pntrb, (size_t)a.m * sizeof(idx_t), hipMemcpyDeviceToHost));
+            FMM_HIP(hipMemcpy(he.data(), a.pntre, (size_t)a.m * sizeof(idx_t), hipMemcpyDeviceToHost));
+            int64_t slots = 0;
+            for (int64_t i = 0; i < a.m; i++) if ((int64_t)he[(size_t)i] > slots) slots = (int64_t)he[(size_t)i];
+            return run_host_sop(a, hb.data(), he.data(), slots, pl, fn);
+         }
+         Args dv;
+         int64_t slots = 0;
+         st = stage_up(a, pl, &dv, &slots);
+         if (st) return st;
+         st = run_host_sop(dv, a.pntrb, a.pntre, slots, pl, fn);
+         if (st) return st;
+         return stage_down(a, dv);
+      }
    }
    if (async) return run_on_device(a, pl, sop_kind, stream);
    if (is_device_pointer(a.z))

@@ -355,6 +355,35 @@ __device__ __forceinline__ float aop_identity(int aop)
    return 0.0f;
 }
 
+// T = VOP(x, y) and s = ROP(x, T) of the general pipeline (reference
+// fusedMM.c:28-202, 721-725); s starts as the edge value (:717).
+template <int L, int R>
+__device__ __forceinline__ float vop_rop(Slice<R> &t, const Slice<R> &xs, const Slice<R> &ys, float edge_val, int vop,
+                                         int rop)
+{
+   switch (vop)
+   {
+      case kVopCopyLhs: t = xs; break;
+      case kVopCopyRhs: t = ys; break;
+      case kVopAdd: map2(t, xs, ys, [](float a, float b) { return a + b; }); break;
+      case kVopSubl: map2(t, xs, ys, [](float a, float b) { return -a + b; }); break;
+      case kVopSubr: map2(t, xs, ys, [](float a, float b) { return a - b; }); break;
+      case kVopMax: map2(t, xs, ys, [](float a, float b) { return a > b ? a : b; }); break;
+      default: map2(t, xs, ys, [](float a, float b) { return a < b ? a : b; }); break;
+   }
+   float scal = edge_val;
+   switch (rop)
+   {
+      case kRopDot: scal = dot_slices<L, R>(xs, t); break;
+      case kRopAddLhs: scal = sum_slice<L, R>(xs); break;
+      case kRopAddRhs: scal = sum_slice<L, R>(t); break;
+      case kRopNormL: scal = dot_slices<L, R>(xs, xs); break;
+      case kRopNormR: scal = dot_slices<L, R>(t, t); break;
+      default: break;
+   }
+   return scal;
+}
+
 // The per-edge pipeline: T = VOP(x, y); s = ROP(x, T); d = SOP(s); T = MOP(d, T);
 // acc = AOP(acc, T).  `xs` is the X[i] slice, `ys` the gathered Y[c] slice.
 template <int L, int R, int OP>
@@ -395,26 +424,7 @@ __device__ __forceinline__ void edge_step(Slice<R> &acc, const Slice<R> &xs, con
       const int vop = imsg & 0xF, rop = imsg & 0xF0, sop = imsg & 0xF00, vsc = imsg & 0xF000,
                 aop = imsg & 0xF0000;
       Slice<R> t;
-      switch (vop)
-      {
-         case kVopCopyLhs: t = xs; break;
-         case kVopCopyRhs: t = ys; break;
-         case kVopAdd: map2(t, xs, ys, [](float a, float b) { return a + b; }); break;
-         case kVopSubl: map2(t, xs, ys, [](float a, float b) { return -a + b; }); break;
-         case kVopSubr: map2(t, xs, ys, [](float a, float b) { return a - b; }); break;
-         case kVopMax: map2(t, xs, ys, [](float a, float b) { return a > b ? a : b; }); break;
-         default: map2(t, xs, ys, [](float a, float b) { return a < b ? a : b; }); break;
-      }
-      float scal = edge_val;
-      switch (rop)
-      {
-         case kRopDot: scal = dot_slices<L, R>(xs, t); break;
-         case kRopAddLhs: scal = sum_slice<L, R>(xs); break;
-         case kRopAddRhs: scal = sum_slice<L, R>(t); break;
-         case kRopNormL: scal = dot_slices<L, R>(xs, xs); break;
-         case kRopNormR: scal = dot_slices<L, R>(t, t); break;
-         default: break;
-      }
+      const float scal = vop_rop<L, R>(t, xs, ys, edge_val, vop, rop);
       const float d = (sop == kSopUdef) ? sop_eval(sop_kind, scal, tab) : scal;
       if (vsc == kVscMul)
       {
@@ -784,6 +794,42 @@ __global__ __launch_bounds__(kBlockThreads) void merge_kernel(const Params<IdxT>
             }
             else if (!p.beta_zero) t = zrow[e] + t;
             zrow[e] = t;
+         }
+      }
+   }
+}
+
+// ---- host-callback SOP, pass 1: s[j] = ROP(X[i], VOP(X[i], Y[c])) for every edge slot ----
+// One wave per row (static stride; this path exists for compatibility, the
+// host evaluates the caller's SOP_UDEF_FUNC on s[] before the accumulate pass).
+template <int V, int L, int R, bool EXACT, int U, typename IdxT>
+__global__ __launch_bounds__(kBlockThreads) void edge_scalar_kernel(const Params<IdxT> p, float *s_out)
+{
+   constexpr int S = 64 / L;
+   const int lane = threadIdx.x & 63;
+   const int sub = lane / L, sl = lane % L;
+   const int64_t wave0 = (int64_t)blockIdx.x * kWavesPerBlock + (threadIdx.x >> 6);
+   const int64_t nwaves = (int64_t)gridDim.x * kWavesPerBlock;
+   const int vop = p.imessage & 0xF, rop = p.imessage & 0xF0;
+   for (int64_t row = wave0; row < p.m; row += nwaves)
+   {
+      const IdxT jb = wave_uniform<IdxT>(p.pntrb[row]);
+      const IdxT je = wave_uniform<IdxT>(p.pntre[row]);
+      Slice<R> xs;
+      load_slice<V, L, R, EXACT>(xs, p.x + row * p.ldx, sl, p.k);
+      for (IdxT j0 = jb; j0 < je; j0 += S * U)
+      {
+#pragma unroll
+         for (int u = 0; u < U; u++)
+         {
+            const IdxT j = j0 + sub + u * S;
+            if (j < je)
+            {
+               Slice<R> ys, t;
+               load_slice<V, L, R, EXACT>(ys, p.y + (int64_t)p.indx[j] * p.ldy, sl, p.k);
+               const float scal = vop_rop<L, R>(t, xs, ys, p.val ? p.val[j] : 0.0f, vop, rop);
+               if (sl == 0) s_out[j] = scal;
+            }
          }
       }
    }

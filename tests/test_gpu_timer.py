@@ -41,3 +41,11 @@ def test_timer_host_pointer_mode(tmp_path):
     assert r.returncode == 0 and "PASSED TEST" in r.stdout, r.stdout
     assert "Filename" not in r.stdout
     assert r.stdout.strip().splitlines()[-1].split(",")[2] == "1000"
+
+
+@pytest.mark.parametrize("bits", [32, 64])
+def test_reference_style_c_caller(bits):
+    """Plain-C program that includes only fusedMM.h, defines SOP_UDEF_FUNC itself
+    and passes host arrays -- the reference's calling convention, untouched."""
+    r = subprocess.run([fbuild.dropin_path(bits)], stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True, timeout=110)
+    assert r.returncode == 0 and "PASSED" in r.stdout, r.stdout
