@@ -225,6 +225,19 @@ __device__ __forceinline__ float sop_eval(int kind, float s, const float *tab)
 
 __device__ __forceinline__ float4 ld4(const float *p) { return *reinterpret_cast<const float4 *>(p); }
 __device__ __forceinline__ void st4(float *p, float4 v) { *reinterpret_cast<float4 *>(p) = v; }
+// Streaming variants for data touched once per call (X rows, Z rows): the
+// non-temporal hint keeps them from displacing gathered Y rows in the caches.
+typedef float v4f_t __attribute__((ext_vector_type(4)));
+__device__ __forceinline__ float4 ld4_stream(const float *p)
+{
+   const v4f_t v = __builtin_nontemporal_load(reinterpret_cast<const v4f_t *>(p));
+   return make_float4(v.x, v.y, v.z, v.w);
+}
+__device__ __forceinline__ void st4_stream(float *p, float4 v)
+{
+   v4f_t t = {v.x, v.y, v.z, v.w};
+   __builtin_nontemporal_store(t, reinterpret_cast<v4f_t *>(p));
+}
 __device__ __forceinline__ float4 zero4() { return make_float4(0.f, 0.f, 0.f, 0.f); }
 
 // One row slice per lane: R float4 registers.
@@ -237,7 +250,7 @@ struct Slice {
 // V == 1: rows that are not 16-byte aligned (K or a leading dimension not a
 // multiple of 4, or an unaligned base): component c of register r holds
 // element (4r+c)*L + sl, loaded and stored 4 bytes at a time.
-template <int V, int L, int R, bool EXACT>
+template <int V, int L, int R, bool EXACT, bool STREAM = false>
 __device__ __forceinline__ void load_slice(Slice<R> &s, const float *row, int sl, int k)
 {
 #pragma unroll
@@ -246,7 +259,7 @@ __device__ __forceinline__ void load_slice(Slice<R> &s, const float *row, int sl
       if (V == 4)
       {
          const int e0 = 4 * (r * L + sl);
-         if (EXACT || e0 < k) s.v[r] = ld4(row + e0);
+         if (EXACT || e0 < k) s.v[r] = STREAM ? ld4_stream(row + e0) : ld4(row + e0);
          else s.v[r] = zero4();
       }
       else
@@ -260,7 +273,7 @@ __device__ __forceinline__ void load_slice(Slice<R> &s, const float *row, int sl
    }
 }
 
-template <int V, int L, int R, bool EXACT>
+template <int V, int L, int R, bool EXACT, bool STREAM = false>
 __device__ __forceinline__ void store_slice(float *row, const Slice<R> &s, int sl, int k)
 {
 #pragma unroll
@@ -269,7 +282,11 @@ __device__ __forceinline__ void store_slice(float *row, const Slice<R> &s, int s
       if (V == 4)
       {
          const int e0 = 4 * (r * L + sl);
-         if (EXACT || e0 < k) st4(row + e0, s.v[r]);
+         if (EXACT || e0 < k)
+         {
+            if (STREAM) st4_stream(row + e0, s.v[r]);
+            else st4(row + e0, s.v[r]);
+         }
       }
       else
       {
@@ -637,7 +654,7 @@ __global__ __launch_bounds__(kBlockThreads) void rows_kernel(const Params<IdxT> 
       }
 
       Slice<R> xs, acc;
-      if (reads_x) load_slice<V, L, R, EXACT>(xs, p.x + row * p.ldx, sl, p.k);
+      if (reads_x) load_slice<V, L, R, EXACT, true>(xs, p.x + row * p.ldx, sl, p.k);
       else
       {
 #pragma unroll
@@ -673,7 +690,7 @@ __global__ __launch_bounds__(kBlockThreads) void rows_kernel(const Params<IdxT> 
             load_slice<V, L, R, EXACT>(zin, zrow, sl, p.k);
             map2(acc, zin, acc, [](float a, float b) { return a + b; });
          }
-         store_slice<V, L, R, EXACT>(zrow, acc, sl, p.k);
+         store_slice<V, L, R, EXACT, true>(zrow, acc, sl, p.k);
       }
    }
    chunk = resolve_claim<IdxT>(p, claimed, cur, nc, nchunks, lane);
@@ -712,7 +729,7 @@ __global__ __launch_bounds__(kBlockThreads) void segments_kernel(const Params<Id
       if (je > re) je = re;
 
       Slice<R> xs, acc;
-      if (reads_x) load_slice<V, L, R, EXACT>(xs, p.x + row * p.ldx, sl, p.k);
+      if (reads_x) load_slice<V, L, R, EXACT, true>(xs, p.x + row * p.ldx, sl, p.k);
       else
       {
 #pragma unroll
