@@ -25,7 +25,9 @@ FLAGS = [
 
 
 def lib_path(index_bits):
-    return os.path.join(HERE, "libfusedmm_amd_i%d.so" % index_bits)
+    """Where the library for INDEXTYPE = int<index_bits>_t lives; FUSEDMM_AMD_LIB_DIR
+    points the loader at another build of it."""
+    return os.path.join(os.environ.get("FUSEDMM_AMD_LIB_DIR", HERE), "libfusedmm_amd_i%d.so" % index_bits)
 
 
 def build_one(index_bits, verbose=False):

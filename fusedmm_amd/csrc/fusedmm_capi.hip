@@ -171,25 +171,32 @@ int pick_shape(int k, bool vec_ok, Shape *s)
       if (k == 32) *s = {4, 8, 1, 1, 8};
       else if (k == 64) *s = {4, 16, 1, 1, 8};
       else if (k == 128) *s = {4, 32, 1, 1, 8};
-      else if (k == 256) *s = {4, 64, 1, 1, 8};
-      else if (k == 512) *s = {4, 64, 2, 1, 4};
+      else if (k == 256) *s = {4, 64, 1, 1, 16};
+      else if (k == 512) *s = {4, 64, 2, 1, 8};
       else if (k <= 32) *s = {4, 8, 1, 0, 8};
       else if (k <= 64) *s = {4, 16, 1, 0, 8};
       else if (k <= 128) *s = {4, 32, 1, 0, 8};
-      else if (k <= 256) *s = {4, 64, 1, 0, 8};
-      else if (k <= 512) *s = {4, 64, 2, 0, 4};
-      else if (k <= 1024) *s = {4, 64, 4, 0, 2};
-      else *s = {4, 64, 8, 0, 1};
+      else if (k <= 256) *s = {4, 64, 1, 0, 16};
+      else if (k <= 512) *s = {4, 64, 2, 0, 8};
+      else if (k <= 1024) *s = {4, 64, 4, 0, 4};
+      else *s = {4, 64, 8, 0, 2};
    }
    else
    {
-      if (k <= 256) *s = {1, 64, 1, 0, 8};
-      else if (k <= 512) *s = {1, 64, 2, 0, 4};
-      else if (k <= 1024) *s = {1, 64, 4, 0, 2};
-      else *s = {1, 64, 8, 0, 1};
+      if (k <= 256) *s = {1, 64, 1, 0, 16};
+      else if (k <= 512) *s = {1, 64, 2, 0, 8};
+      else if (k <= 1024) *s = {1, 64, 4, 0, 4};
+      else *s = {1, 64, 8, 0, 2};
    }
    return FUSEDMM_SUCCESS_RETURN;
 }
+
+// (V, L, R, exact, U) of every kernel instance; pick_shape() returns one of these.
+#define FMM_SHAPES(X) \
+   X(4, 8, 1, 1, 8) X(4, 16, 1, 1, 8) X(4, 32, 1, 1, 8) X(4, 64, 1, 1, 16) X(4, 64, 2, 1, 8) \
+   X(4, 8, 1, 0, 8) X(4, 16, 1, 0, 8) X(4, 32, 1, 0, 8) X(4, 64, 1, 0, 16) X(4, 64, 2, 0, 8) \
+   X(4, 64, 4, 0, 4) X(4, 64, 8, 0, 2) \
+   X(1, 64, 1, 0, 16) X(1, 64, 2, 0, 8) X(1, 64, 4, 0, 4) X(1, 64, 8, 0, 2)
 
 struct Launch {
    int num_cu, blocks_per_cu;
@@ -197,15 +204,15 @@ struct Launch {
    hipEvent_t *ev;   // 4 events or nullptr
 };
 
-template <int V, int L, int R, bool EXACT, int OP, int U>
+template <int V, int L, int R, bool EXACT, int OP, int SOPK, int U>
 int launch_instance(const Params<idx_t> &p, const Launch &l)
 {
    // persistent grids: as many blocks as stay resident, each wave strides over rows
    static int occ_rows = 0, occ_segs = 0;
    if (occ_rows == 0)
    {
-      FMM_HIP(hipOccupancyMaxActiveBlocksPerMultiprocessor(&occ_rows, rows_kernel<V, L, R, EXACT, OP, U, idx_t>, kBlockThreads, 0));
-      FMM_HIP(hipOccupancyMaxActiveBlocksPerMultiprocessor(&occ_segs, segments_kernel<V, L, R, EXACT, OP, U, idx_t>, kBlockThreads, 0));
+      FMM_HIP(hipOccupancyMaxActiveBlocksPerMultiprocessor(&occ_rows, rows_kernel<V, L, R, EXACT, OP, SOPK, U, idx_t>, kBlockThreads, 0));
+      FMM_HIP(hipOccupancyMaxActiveBlocksPerMultiprocessor(&occ_segs, segments_kernel<V, L, R, EXACT, OP, SOPK, U, idx_t>, kBlockThreads, 0));
       if (occ_rows < 1) occ_rows = 1;
       if (occ_segs < 1) occ_segs = 1;
    }
@@ -216,36 +223,24 @@ int launch_instance(const Params<idx_t> &p, const Launch &l)
    pr.row_counters = (gr * kWavesPerBlock >= kRowCounters) ? kRowCounters : 1;
    const int64_t gs = (int64_t)l.num_cu * (l.blocks_per_cu > 0 ? l.blocks_per_cu : occ_segs);
    if (l.ev) FMM_HIP(hipEventRecord(l.ev[0], l.stream));
-   hipLaunchKernelGGL((rows_kernel<V, L, R, EXACT, OP, U, idx_t>), dim3((unsigned int)gr), dim3(kBlockThreads), 0, l.stream, pr);
+   hipLaunchKernelGGL((rows_kernel<V, L, R, EXACT, OP, SOPK, U, idx_t>), dim3((unsigned int)gr), dim3(kBlockThreads), 0, l.stream, pr);
    if (l.ev) FMM_HIP(hipEventRecord(l.ev[1], l.stream));
-   hipLaunchKernelGGL((segments_kernel<V, L, R, EXACT, OP, U, idx_t>), dim3((unsigned int)gs), dim3(kBlockThreads), 0, l.stream, p);
+   hipLaunchKernelGGL((segments_kernel<V, L, R, EXACT, OP, SOPK, U, idx_t>), dim3((unsigned int)gs), dim3(kBlockThreads), 0, l.stream, p);
    if (l.ev) FMM_HIP(hipEventRecord(l.ev[2], l.stream));
    hipLaunchKernelGGL((merge_kernel<idx_t>), dim3((unsigned int)(l.num_cu * 2)), dim3(kBlockThreads), 0, l.stream, p, (int)(OP == OP_GENERIC));
    if (l.ev) FMM_HIP(hipEventRecord(l.ev[3], l.stream));
    return hip_status(hipGetLastError(), "kernel launch");
 }
 
-template <int OP>
+// SOPK >= 0: the SOP body is fixed at compile time (the three the reference's
+// benchmarks use: sigmoid on the dot tuple, t-dist and FR on the distance
+// tuple); SOPK == -1: switched at run time on Params::sop_kind.
+template <int OP, int SOPK>
 int launch_op(const Params<idx_t> &p, const Shape &s, const Launch &l)
 {
 #define FMM_CASE(V_, L_, R_, X_, U_) \
-   if (s.V == V_ && s.L == L_ && s.R == R_ && s.exact == X_) return launch_instance<V_, L_, R_, (X_ != 0), OP, U_>(p, l);
-   FMM_CASE(4, 8, 1, 1, 8)
-   FMM_CASE(4, 16, 1, 1, 8)
-   FMM_CASE(4, 32, 1, 1, 8)
-   FMM_CASE(4, 64, 1, 1, 8)
-   FMM_CASE(4, 64, 2, 1, 4)
-   FMM_CASE(4, 8, 1, 0, 8)
-   FMM_CASE(4, 16, 1, 0, 8)
-   FMM_CASE(4, 32, 1, 0, 8)
-   FMM_CASE(4, 64, 1, 0, 8)
-   FMM_CASE(4, 64, 2, 0, 4)
-   FMM_CASE(4, 64, 4, 0, 2)
-   FMM_CASE(4, 64, 8, 0, 1)
-   FMM_CASE(1, 64, 1, 0, 8)
-   FMM_CASE(1, 64, 2, 0, 4)
-   FMM_CASE(1, 64, 4, 0, 2)
-   FMM_CASE(1, 64, 8, 0, 1)
+   if (s.V == V_ && s.L == L_ && s.R == R_ && s.exact == X_) return launch_instance<V_, L_, R_, (X_ != 0), OP, SOPK, U_>(p, l);
+   FMM_SHAPES(FMM_CASE)
 #undef FMM_CASE
    return FUSEDMM_FAIL_RETURN;
 }
@@ -397,11 +392,16 @@ int run_on_device(const Args &a, const Plan &pl, int sop_kind, hipStream_t strea
 
    switch (pl.op)
    {
-      case OP_GCN: return launch_op<OP_GCN>(p, sh, l);
-      case OP_SPMM: return launch_op<OP_SPMM>(p, sh, l);
-      case OP_DOT: return launch_op<OP_DOT>(p, sh, l);
-      case OP_DIST: return launch_op<OP_DIST>(p, sh, l);
-      default: return launch_op<OP_GENERIC>(p, sh, l);
+      case OP_GCN: return launch_op<OP_GCN, -1>(p, sh, l);
+      case OP_SPMM: return launch_op<OP_SPMM, -1>(p, sh, l);
+      case OP_DOT:
+         if (sop_kind == SOP_SIGMOID) return launch_op<OP_DOT, SOP_SIGMOID>(p, sh, l);
+         return launch_op<OP_DOT, -1>(p, sh, l);
+      case OP_DIST:
+         if (sop_kind == SOP_TDIST) return launch_op<OP_DIST, SOP_TDIST>(p, sh, l);
+         if (sop_kind == SOP_FR) return launch_op<OP_DIST, SOP_FR>(p, sh, l);
+         return launch_op<OP_DIST, -1>(p, sh, l);
+      default: return launch_op<OP_GENERIC, -1>(p, sh, l);
    }
 }
 
@@ -535,13 +535,10 @@ int run_host_sop(const Args &a, const idx_t *h_pb, const idx_t *h_pe, int64_t sl
    p.pntrb = a.pntrb; p.pntre = a.pntre; p.indx = a.indx; p.val = a.val;
    p.x = a.x ? a.x : a.y;   // tuples that never read X still index it; any valid row will do
    p.y = a.y; p.m = a.m; p.ldx = a.x ? a.ldx : 0; p.ldy = a.ldy; p.k = (int)a.k; p.imessage = a.imessage;
-#define FMM_CASE(V_, L_, R_, X_, U_) \
-   if (sh.V == V_ && sh.L == L_ && sh.R == R_ && sh.exact == X_) st = launch_edge_scalar<V_, L_, R_, (X_ != 0), U_>(p, d_s, d->num_cu); else
-   FMM_CASE(4, 8, 1, 1, 8) FMM_CASE(4, 16, 1, 1, 8) FMM_CASE(4, 32, 1, 1, 8) FMM_CASE(4, 64, 1, 1, 8)
-   FMM_CASE(4, 64, 2, 1, 4) FMM_CASE(4, 8, 1, 0, 8) FMM_CASE(4, 16, 1, 0, 8) FMM_CASE(4, 32, 1, 0, 8)
-   FMM_CASE(4, 64, 1, 0, 8) FMM_CASE(4, 64, 2, 0, 4) FMM_CASE(4, 64, 4, 0, 2) FMM_CASE(4, 64, 8, 0, 1)
-   FMM_CASE(1, 64, 1, 0, 8) FMM_CASE(1, 64, 2, 0, 4) FMM_CASE(1, 64, 4, 0, 2) FMM_CASE(1, 64, 8, 0, 1)
    st = FUSEDMM_FAIL_RETURN;
+#define FMM_CASE(V_, L_, R_, X_, U_) \
+   if (sh.V == V_ && sh.L == L_ && sh.R == R_ && sh.exact == X_) st = launch_edge_scalar<V_, L_, R_, (X_ != 0), U_>(p, d_s, d->num_cu);
+   FMM_SHAPES(FMM_CASE)
 #undef FMM_CASE
    if (st) return st;
    std::vector<float> hs((size_t)slots);

@@ -199,7 +199,11 @@ __device__ __forceinline__ float sop_eval(int kind, float s, const float *tab)
          else if (s < -5.0f) t = 0.0f;
          else
          {
-            int idx = (int)(((double)s + 5.0) * 2048.0 / 10.0);
+            // The reference evaluates ((double)s + 5.0) * 2048 / 10.0.  One multiply by
+            // 204.8 truncates to the same integer for every float in [-5, 5]
+            // (checked exhaustively over all 2 168 455 170 of them on the CPU), and
+            // spares a double-precision division per edge.
+            int idx = (int)(((double)s + 5.0) * 204.8);
             idx = idx > kSigmoidTableSize - 1 ? kSigmoidTableSize - 1 : idx;
             t = tab[idx];
          }
@@ -467,36 +471,91 @@ __device__ __forceinline__ void edge_step(Slice<R> &acc, const Slice<R> &xs, con
    }
 }
 
-// Edges [jb, je) of one row, dealt round-robin to the sub-waves, U gathers in
+// 64 consecutive edge slots of a row, one per lane: column id and edge value.
+template <typename IdxT>
+struct EdgeChunk {
+   IdxT col;
+   float val;
+};
+
+template <int OP, typename IdxT>
+__device__ __forceinline__ void load_chunk(EdgeChunk<IdxT> &c, const Params<IdxT> &p, IdxT j0, IdxT je, int lane)
+{
+   const IdxT j = j0 + lane;
+   c.col = 0;
+   c.val = 0.0f;
+   if (j < je)
+   {
+      c.col = p.indx[j];
+      if ((OP == OP_SPMM || OP == OP_GENERIC) && p.val) c.val = p.val[j];
+   }
+}
+
+// Entry `e` of a chunk.  Whole-wave rows (L == 64): e is wave-uniform and the
+// value lands in a scalar register (v_readlane), so the gather address is
+// scalar too.  Narrower sub-waves each want a different entry: ds_bpermute.
+template <int L>
+__device__ __forceinline__ int32_t chunk_entry(int32_t v, int e)
+{
+   if (L == 64) return __builtin_amdgcn_readlane(v, e);
+   return __builtin_amdgcn_ds_bpermute(e << 2, v);
+}
+template <int L>
+__device__ __forceinline__ int64_t chunk_entry(int64_t v, int e)
+{
+   const int lo = chunk_entry<L>((int32_t)(v & 0xFFFFFFFFll), e);
+   const int hi = chunk_entry<L>((int32_t)(v >> 32), e);
+   return ((int64_t)hi << 32) | (uint32_t)lo;
+}
+template <int L>
+__device__ __forceinline__ float chunk_entry(float v, int e)
+{
+   return as_f(chunk_entry<L>(as_i(v), e));
+}
+
+// Edges [jb, je) of one row, dealt round-robin to the sub-waves.  Column ids
+// (and edge values) are fetched 64 at a time with one coalesced load per
+// array, the next 64 while the current ones are being used; U gathers are in
 // flight per sub-wave.  All lanes of the wave call this with the same jb, je.
-template <int V, int L, int R, bool EXACT, int OP, int U, typename IdxT>
+template <int V, int L, int R, bool EXACT, int OP, int SOPK, int U, typename IdxT>
 __device__ __forceinline__ void walk_edges(Slice<R> &acc, const Slice<R> &xs, const Params<IdxT> &p,
-                                           IdxT jb, IdxT je, int sub, int sl, const float *tab)
+                                           IdxT jb, IdxT je, int lane, const float *tab)
 {
    constexpr int S = 64 / L;
-   for (IdxT j0 = jb; j0 < je; j0 += S * U)
+   const int sub = (L == 64) ? 0 : lane / L, sl = (L == 64) ? lane : lane % L;
+   const int sop_kind = SOPK >= 0 ? SOPK : p.sop_kind;
+   if (jb >= je) return;
+   EdgeChunk<IdxT> cur;
+   load_chunk<OP, IdxT>(cur, p, jb, je, lane);
+   for (IdxT j0 = jb; j0 < je; j0 += 64)
    {
-      IdxT col[U];
-      float ev[U];
-      Slice<R> ys[U];
-#pragma unroll
-      for (int u = 0; u < U; u++)
+      EdgeChunk<IdxT> nxt;
+      nxt.col = 0;
+      nxt.val = 0.0f;
+      if (j0 + 64 < je) load_chunk<OP, IdxT>(nxt, p, j0 + 64, je, lane);
+      const int n = (je - j0) < 64 ? (int)(je - j0) : 64;
+      for (int b0 = 0; b0 < n; b0 += S * U)
       {
-         const IdxT j = j0 + sub + u * S;
-         col[u] = -1;
-         ev[u] = 0.0f;
-         if (j < je)
+         IdxT col[U];
+         float ev[U];
+         bool ok[U];
+         Slice<R> ys[U];
+#pragma unroll
+         for (int u = 0; u < U; u++)
          {
-            col[u] = p.indx[j];
-            if (OP == OP_SPMM || OP == OP_GENERIC) ev[u] = p.val ? p.val[j] : 0.0f;
+            const int e = b0 + u * S + sub;     // L == 64: sub == 0, e is uniform
+            ok[u] = e < n;
+            col[u] = chunk_entry<L>(cur.col, e & 63);
+            ev[u] = (OP == OP_SPMM || OP == OP_GENERIC) ? chunk_entry<L>(cur.val, e & 63) : 0.0f;
          }
+#pragma unroll
+         for (int u = 0; u < U; u++)
+            if (ok[u]) load_slice<V, L, R, EXACT>(ys[u], p.y + (int64_t)col[u] * p.ldy, sl, p.k);
+#pragma unroll
+         for (int u = 0; u < U; u++)
+            if (ok[u]) edge_step<L, R, OP>(acc, xs, ys[u], ev[u], sop_kind, p.imessage, tab);
       }
-#pragma unroll
-      for (int u = 0; u < U; u++)
-         if (col[u] >= 0) load_slice<V, L, R, EXACT>(ys[u], p.y + (int64_t)col[u] * p.ldy, sl, p.k);
-#pragma unroll
-      for (int u = 0; u < U; u++)
-         if (col[u] >= 0) edge_step<L, R, OP>(acc, xs, ys[u], ev[u], p.sop_kind, p.imessage, tab);
+      cur = nxt;
    }
 }
 
@@ -575,13 +634,13 @@ __device__ __forceinline__ int64_t resolve_claim(const Params<IdxT> &p, unsigned
 }
 
 // ---- kernel 1: one wavefront per row, heavy rows queued -------------------------
-template <int V, int L, int R, bool EXACT, int OP, int U, typename IdxT>
+template <int V, int L, int R, bool EXACT, int OP, int SOPK, int U, typename IdxT>
 __global__ __launch_bounds__(kBlockThreads) void rows_kernel(const Params<IdxT> p)
 {
    constexpr int S = 64 / L;
    __shared__ float lds_tab[(OP >= OP_DOT) ? kSigmoidTableSize : 1];
    const bool uses_sop = (OP == OP_DOT || OP == OP_DIST || (OP == OP_GENERIC && (p.imessage & 0xF00) == kSopUdef));
-   const float *tab = stage_table(p.sigmoid_table, lds_tab, (OP >= OP_DOT) && uses_sop && p.sop_kind == SOP_SIGMOID);
+   const float *tab = stage_table(p.sigmoid_table, lds_tab, (OP >= OP_DOT) && uses_sop && (SOPK >= 0 ? SOPK : p.sop_kind) == SOP_SIGMOID);
 
    const int lane = threadIdx.x & 63;
    const int sub = lane / L, sl = lane % L;
@@ -679,7 +738,7 @@ __global__ __launch_bounds__(kBlockThreads) void rows_kernel(const Params<IdxT> 
          for (int r = 0; r < R; r++) acc.v[r] = zero4();
       }
 
-      walk_edges<V, L, R, EXACT, OP, U, IdxT>(acc, xs, p, jb, je, sub, sl, tab);
+      walk_edges<V, L, R, EXACT, OP, SOPK, U, IdxT>(acc, xs, p, jb, je, lane, tab);
       merge_subwaves<L, R, OP>(acc, p.imessage);
 
       if (sub == 0)
@@ -698,7 +757,7 @@ __global__ __launch_bounds__(kBlockThreads) void rows_kernel(const Params<IdxT> 
 }
 
 // ---- kernel 2: one wavefront per queued edge segment -> partial Z -----------------
-template <int V, int L, int R, bool EXACT, int OP, int U, typename IdxT>
+template <int V, int L, int R, bool EXACT, int OP, int SOPK, int U, typename IdxT>
 __global__ __launch_bounds__(kBlockThreads) void segments_kernel(const Params<IdxT> p)
 {
    __shared__ float lds_tab[(OP >= OP_DOT) ? kSigmoidTableSize : 1];
@@ -706,7 +765,7 @@ __global__ __launch_bounds__(kBlockThreads) void segments_kernel(const Params<Id
    if (nseg > p.cap_seg) nseg = p.cap_seg;   // rows beyond the cap were done inline
    if (nseg == 0) return;
    const bool uses_sop = (OP == OP_DOT || OP == OP_DIST || (OP == OP_GENERIC && (p.imessage & 0xF00) == kSopUdef));
-   const float *tab = stage_table(p.sigmoid_table, lds_tab, (OP >= OP_DOT) && uses_sop && p.sop_kind == SOP_SIGMOID);
+   const float *tab = stage_table(p.sigmoid_table, lds_tab, (OP >= OP_DOT) && uses_sop && (SOPK >= 0 ? SOPK : p.sop_kind) == SOP_SIGMOID);
 
    const int lane = threadIdx.x & 63;
    const int sub = lane / L, sl = lane % L;
@@ -739,7 +798,7 @@ __global__ __launch_bounds__(kBlockThreads) void segments_kernel(const Params<Id
 #pragma unroll
       for (int r = 0; r < R; r++) acc.v[r] = make_float4(id, id, id, id);
 
-      walk_edges<V, L, R, EXACT, OP, U, IdxT>(acc, xs, p, jb, je, sub, sl, tab);
+      walk_edges<V, L, R, EXACT, OP, SOPK, U, IdxT>(acc, xs, p, jb, je, lane, tab);
       merge_subwaves<L, R, OP>(acc, p.imessage);
 
       if (sub == 0) store_slice<V, L, R, EXACT>(p.partial + (int64_t)q * p.kpad, acc, sl, p.k);

@@ -200,6 +200,29 @@ float orc_gpu_dot(const float *x, const float *y, int64_t K, int V, int L, int d
    return p[0];
 }
 
+/* Counts the floats v in [-5, 5] for which the reference's bin expression
+ * (orc_sigmoid_bin, a double division by 10.0) and the single multiply
+ * (int)(((double)v + 5.0) * 204.8) disagree.  The GPU kernels use the multiply;
+ * the count must be zero.  Visits every float bit pattern. */
+int64_t orc_count_bin_formula_mismatches(int64_t *visited)
+{
+   int64_t bad = 0, seen = 0;
+#pragma omp parallel for reduction(+ : bad, seen) schedule(static)
+   for (int64_t u = 0; u < ((int64_t)1 << 32); u++)
+   {
+      uint32_t bits = (uint32_t)u;
+      float v;
+      memcpy(&v, &bits, sizeof(v));
+      if (!(v >= -5.0f && v <= 5.0f)) continue;
+      seen++;
+      int want = (int)(((double)v + ORC_SM_BOUND) * ORC_SM_TABLE_SIZE / (2.0 * ORC_SM_BOUND));
+      int got = (int)(((double)v + 5.0) * 204.8);
+      bad += (want != got);
+   }
+   if (visited) *visited = seen;
+   return bad;
+}
+
 int orc_max_threads(void)
 {
 #ifdef _OPENMP
