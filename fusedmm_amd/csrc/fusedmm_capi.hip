@@ -371,7 +371,7 @@ int run_on_device(const Args &a, const Plan &pl, int sop_kind, hipStream_t strea
    p.cap_heavy = (unsigned int)cap_heavy;
    p.cap_seg = (unsigned int)cap_seg;
 
-   FMM_HIP(hipMemsetAsync(d->ctr, 0, sizeof(Counters), stream));
+   hipLaunchKernelGGL(reset_counters_kernel, dim3(1), dim3(kBlockThreads), 0, stream, d->ctr);
 
    Launch l;
    l.num_cu = d->num_cu;

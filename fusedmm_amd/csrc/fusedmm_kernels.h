@@ -911,6 +911,14 @@ __global__ __launch_bounds__(kBlockThreads) void edge_scalar_kernel(const Params
    }
 }
 
+// Clears the queue and claim counters before each call.  A kernel rather than a
+// memset so that callers may capture the stream entry point in a HIP graph.
+__global__ __launch_bounds__(kBlockThreads) void reset_counters_kernel(Counters *c)
+{
+   unsigned int *w = reinterpret_cast<unsigned int *>(c);
+   for (unsigned int i = threadIdx.x; i < sizeof(Counters) / sizeof(unsigned int); i += kBlockThreads) w[i] = 0u;
+}
+
 // Plain 16-byte copy of known size: the yardstick the HBM traffic counters
 // (FETCH_SIZE / WRITE_SIZE) of the kernels above are scaled by.
 __global__ __launch_bounds__(kBlockThreads) void copy_probe_kernel(float4 *dst, const float4 *src, int64_t n16)

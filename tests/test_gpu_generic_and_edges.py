@@ -175,3 +175,43 @@ def test_golden_ops_on_gpu(oracle, bits):
                 if t == "s":
                     extra = extra + checks.sigmoid_flip_slack(oracle.table(), g, X, Y)[0]
                 checks.assert_close(Z, want, rtol, atol, extra, "%s %s k=%d" % (gname, t, k))
+
+
+def test_stream_entry_can_be_captured_in_a_hip_graph(oracle):
+    """fusedMM_csr_stream enqueues kernels only (no memset, no allocation once the
+    work queues exist): a caller may capture it and replay it.  Every replay is
+    checked against the eager result, with eager work in between; the graph has
+    split rows, so all three kernels and the queue reset are replayed."""
+    import torch
+    g = graphs.ragged(32, rows=200, cols=3000, hub_deg=5000)
+    k = 128
+    X = graphs.features(g["rows"], k, 3, -0.5, 0.5, 1)
+    Y = graphs.features(g["cols"], k, 3, -0.5, 0.5, 2)
+    dev = torch.device("cuda:0")
+    t = lambda a: torch.from_numpy(np.ascontiguousarray(a)).to(dev)
+    val, indx, pb, pe, dX, dY = t(g["val"]), t(g["indx"]), t(g["pntrb"]), t(g["pntre"]), t(X), t(Y)
+    gpu_api.set_kind(SOP_NAMES["sigmoid"], 32)
+
+    def enqueue(Z):
+        rc = fa.fusedMM_csr(fa.MSG_SIGMOID, g["rows"], g["cols"], k, 1.0, g["nnz"], g["rows"], g["cols"], val, indx,
+                            pb, pe, dX, k, dY, k, 0.0, Z, k, stream=torch.cuda.current_stream().cuda_stream)
+        assert rc == 0
+
+    Zeager = torch.zeros((g["rows"], k), device=dev)
+    enqueue(Zeager)                                   # also sizes the work queues
+    torch.cuda.synchronize()
+    assert gpu_api.last_split(32)[1] > 0
+    Zg = torch.full((g["rows"], k), 9.0, device=dev)
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        enqueue(Zg)
+    for rep in range(4):
+        Zg.fill_(float(rep))
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(Zg, Zeager), rep
+        dY2 = dY * 2.0                                # eager work between replays
+        Ze2 = torch.zeros_like(Zeager)
+        rc = fa.fusedMM_csr(fa.MSG_SIGMOID, g["rows"], g["cols"], k, 1.0, g["nnz"], g["rows"], g["cols"], val, indx,
+                            pb, pe, dX, k, dY2, k, 0.0, Ze2, k)
+        assert rc == 0
