@@ -32,7 +32,7 @@ SOP_KIND_HOST, SOP_KIND_IDENTITY, SOP_KIND_SIGMOID, SOP_KIND_TDIST, SOP_KIND_FR,
 SUCCESS, FAIL, VOP_FAIL, ROP_FAIL, AOP_FAIL, SOP_FAIL, VSC_FAIL = 0, 1, 2, 4, 8, 16, 32
 NOT_ENOUGH_MEM, UNDEFINED_USER_FUNCTION, NO_OPT_IMPL = -1, 64, 128
 
-EXPORTS = ("fusedMM_csr", "fusedMM_csr_stream", "sgfusedMM_csr", "fusedMM_amd_index_bytes",
+EXPORTS = ("fusedMM_csr", "fusedMM_csr_stream", "fusedMM_amd_index_bytes", "fusedMM_amd_value_bytes",
            "fusedMM_amd_set_sop_kind", "fusedMM_amd_get_sop_kind", "fusedMM_amd_set_sop_callback",
            "fusedMM_amd_set_opt", "fusedMM_amd_set_split", "fusedMM_amd_timing",
            "fusedMM_amd_timing_summary", "fusedMM_amd_last_split", "fusedMM_amd_copy_probe",
@@ -41,10 +41,12 @@ EXPORTS = ("fusedMM_csr", "fusedMM_csr_stream", "sgfusedMM_csr", "fusedMM_amd_in
 _libs = {}
 
 
-def load(index_bits=32):
-    """dlopen the library for INDEXTYPE = int<index_bits>_t and declare its signatures."""
-    if index_bits in _libs:
-        return _libs[index_bits]
+def load(index_bits=32, value_bits=32):
+    """dlopen the library for INDEXTYPE = int<index_bits>_t and VALUETYPE = float
+    (value_bits 32) or double (64), and declare its signatures."""
+    key = (index_bits, value_bits)
+    if key in _libs:
+        return _libs[key]
     # One HIP runtime per process: when PyTorch is present its bundled
     # libamdhip64 (same SONAME as ROCm's) must be mapped first, so that this
     # library binds to it and device addresses and streams can be shared.
@@ -52,20 +54,23 @@ def load(index_bits=32):
         import torch  # noqa: F401
     except ImportError:
         pass
-    path = lib_path(index_bits)
+    path = lib_path(index_bits, value_bits)
     if not os.path.exists(path):
         raise OSError("%s is not built; run `python -m fusedmm_amd.build`" % path)
     lib = C.CDLL(path)
     it = C.c_int32 if index_bits == 32 else C.c_int64
+    vt = C.c_float if value_bits == 32 else C.c_double
     vp = C.c_void_p
-    csr = [C.c_int32, it, it, it, C.c_float, it, it, it, vp, vp, vp, vp, vp, it, vp, it, C.c_float, vp, it]
+    csr = [C.c_int32, it, it, it, vt, it, it, it, vp, vp, vp, vp, vp, it, vp, it, vt, vp, it]
     lib.fusedMM_csr.argtypes = csr
     lib.fusedMM_csr.restype = C.c_int
     lib.fusedMM_csr_stream.argtypes = csr + [vp]
     lib.fusedMM_csr_stream.restype = C.c_int
-    lib.sgfusedMM_csr.argtypes = [C.c_char] + csr[1:]
-    lib.sgfusedMM_csr.restype = None
+    gf = lib.sgfusedMM_csr if value_bits == 32 else lib.dgfusedMM_csr   # kernels.h:17-37 of the reference
+    gf.argtypes = [C.c_char] + csr[1:]
+    gf.restype = None
     lib.fusedMM_amd_index_bytes.restype = C.c_int
+    lib.fusedMM_amd_value_bytes.restype = C.c_int
     lib.fusedMM_amd_set_sop_kind.argtypes = [C.c_int]
     lib.fusedMM_amd_set_sop_kind.restype = C.c_int
     lib.fusedMM_amd_get_sop_kind.restype = C.c_int
@@ -81,7 +86,8 @@ def load(index_bits=32):
     lib.fusedMM_amd_copy_probe.argtypes = [vp, vp, C.c_int64, vp]
     lib.fusedMM_amd_copy_probe.restype = C.c_int
     assert lib.fusedMM_amd_index_bytes() * 8 == index_bits
-    _libs[index_bits] = lib
+    assert lib.fusedMM_amd_value_bytes() * 8 == value_bits
+    _libs[key] = lib
     return lib
 
 
@@ -97,11 +103,11 @@ def _addr(a):
 
 
 def fusedMM_csr(imessage, m, n, k, alpha, nnz, rows, cols, val, indx, pntrb, pntre, x, ldx, y, ldy, beta, z, ldz,
-                index_bits=32, stream=None):
+                index_bits=32, stream=None, value_bits=32):
     """Same argument list as the C entry point (include/fusedMM.h).  Operands
     are numpy arrays (host memory) or torch tensors / integer addresses (device
     memory).  With `stream` (an integer hipStream_t) the call is asynchronous."""
-    lib = load(index_bits)
+    lib = load(index_bits, value_bits)
     args = [imessage, m, n, k, alpha, nnz, rows, cols, _addr(val), _addr(indx), _addr(pntrb), _addr(pntre),
             _addr(x), ldx, _addr(y), ldy, beta, _addr(z), ldz]
     if stream is None:

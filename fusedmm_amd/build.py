@@ -24,22 +24,27 @@ FLAGS = [
 ]
 
 
-def lib_path(index_bits):
+def lib_name(index_bits, value_bits=32):
+    """libfusedmm_amd_i<bits>.so for float (the reference's default), libfusedmm_amd_d_i<bits>.so for double."""
+    return "libfusedmm_amd_%si%d.so" % ("d_" if value_bits == 64 else "", index_bits)
+
+
+def lib_path(index_bits, value_bits=32):
     """Where the library for INDEXTYPE = int<index_bits>_t lives; FUSEDMM_AMD_LIB_DIR
     points the loader at another build of it."""
-    return os.path.join(os.environ.get("FUSEDMM_AMD_LIB_DIR", HERE), "libfusedmm_amd_i%d.so" % index_bits)
+    return os.path.join(os.environ.get("FUSEDMM_AMD_LIB_DIR", HERE), lib_name(index_bits, value_bits))
 
 
-def build_one(index_bits, verbose=False):
-    out = lib_path(index_bits)
-    cmd = [HIPCC] + FLAGS + ["-DINDEXTYPE=int%d_t" % index_bits,
-                             os.path.join(CSRC, "fusedmm_capi.hip"), "-o", out, "-ldl"]
+def build_one(index_bits, value_bits=32, verbose=False):
+    out = os.path.join(HERE, lib_name(index_bits, value_bits))
+    cmd = [HIPCC] + FLAGS + ["-DINDEXTYPE=int%d_t" % index_bits] + (["-DDREAL"] if value_bits == 64 else []) + \
+          [os.path.join(CSRC, "fusedmm_capi.hip"), "-o", out, "-ldl"]
     if verbose:
         print(" ".join(cmd), flush=True)
     r = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
     if r.returncode != 0:
         sys.stderr.write(r.stdout)
-        raise RuntimeError("hipcc failed for int%d" % index_bits)
+        raise RuntimeError("hipcc failed for int%d / %d-bit values" % (index_bits, value_bits))
     return out
 
 
@@ -81,8 +86,8 @@ def build_timer(index_bits, verbose=False):
 
 
 def build_all(verbose=False):
-    with ThreadPoolExecutor(2) as ex:
-        libs = list(ex.map(lambda b: build_one(b, verbose), (32, 64)))
+    with ThreadPoolExecutor(4) as ex:
+        libs = list(ex.map(lambda a: build_one(a[0], a[1], verbose), ((32, 32), (64, 32), (32, 64), (64, 64))))
         exes = list(ex.map(lambda b: build_timer(b, verbose), (32, 64)))
     return libs + exes
 

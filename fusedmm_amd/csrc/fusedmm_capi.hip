@@ -19,7 +19,12 @@
 #ifndef INDEXTYPE
 #error "compile with -DINDEXTYPE=int32_t or -DINDEXTYPE=int64_t"
 #endif
+#ifdef DREAL          /* the reference's switch for double precision (fusedMM.c:9-13) */
+#define FMM_DOUBLE 1
+#define VALUETYPE double
+#else
 #define VALUETYPE float
+#endif
 #include "../../include/fusedMM.h"
 #include "../../include/fusedmm_amd.h"
 #include "fusedmm_kernels.h"
@@ -28,6 +33,8 @@ namespace {
 
 using namespace fmm;
 typedef INDEXTYPE idx_t;
+typedef VALUETYPE val_t;
+constexpr size_t kValBytes = sizeof(val_t);
 
 #define FMM_LOG(...)                                   \
    do {                                                \
@@ -61,7 +68,7 @@ struct Buffer {
 struct DeviceState {
    bool ready = false;
    int num_cu = 0;
-   float *sigmoid_table = nullptr;
+   val_t *sigmoid_table = nullptr;
    Counters *ctr = nullptr;
    Buffer heavy, segs, partial;
    Buffer stage[8];           // host-pointer mode: pntrb, pntre, indx, val, x, y, z, spare
@@ -109,16 +116,23 @@ void read_env_once()
 }
 
 // The 2048-entry sigmoid table, built with the expressions of the reference's
-// tester (test/fusedMMtime.cpp:594-604): x is a float, exp is the float
-// overload, 1 + e is a float sum, the quotient is formed in double.
-void build_sigmoid_table(float *t)
+// tester (test/fusedMMtime.cpp:594-604, a C++ file: exp() resolves to the
+// overload of VALUETYPE).  Single precision: x is a float, exp is expf, 1 + e is
+// a float sum, the quotient is formed in double and rounded.  Double precision:
+// everything is double.
+void build_sigmoid_table(val_t *t)
 {
    for (int i = 0; i < kSigmoidTableSize; i++)
    {
+#ifdef FMM_DOUBLE
+      double x = 2.0 * 5.0 * i / kSigmoidTableSize - 5.0;
+      t[i] = 1.0 / (1 + exp(-x));
+#else
       float x = (float)(2.0 * 5.0 * i / kSigmoidTableSize - 5.0);
       float e = expf(-x);
       float denom = 1 + e;
       t[i] = (float)(1.0 / (double)denom);
+#endif
    }
 }
 
@@ -144,7 +158,7 @@ int device_state(DeviceState **out)
       hipDeviceProp_t prop;
       FMM_HIP(hipGetDeviceProperties(&prop, dev));
       d.num_cu = prop.multiProcessorCount > 0 ? prop.multiProcessorCount : 256;
-      float host_tab[kSigmoidTableSize];
+      val_t host_tab[kSigmoidTableSize];
       build_sigmoid_table(host_tab);
       FMM_HIP(hipMalloc((void **)&d.sigmoid_table, sizeof(host_tab)));
       FMM_HIP(hipMemcpy(d.sigmoid_table, host_tab, sizeof(host_tab), hipMemcpyHostToDevice));
@@ -192,11 +206,18 @@ int pick_shape(int k, bool vec_ok, Shape *s)
 }
 
 // (V, L, R, exact, U) of every kernel instance; pick_shape() returns one of these.
+// U (gathers in flight per sub-wave) is halved in double precision: same bytes in flight.
+#ifdef FMM_DOUBLE
+#define FMM_U(u) ((u) / 2)
+#else
+#define FMM_U(u) (u)
+#endif
 #define FMM_SHAPES(X) \
-   X(4, 8, 1, 1, 8) X(4, 16, 1, 1, 8) X(4, 32, 1, 1, 8) X(4, 64, 1, 1, 16) X(4, 64, 2, 1, 8) \
-   X(4, 8, 1, 0, 8) X(4, 16, 1, 0, 8) X(4, 32, 1, 0, 8) X(4, 64, 1, 0, 16) X(4, 64, 2, 0, 8) \
-   X(4, 64, 4, 0, 4) X(4, 64, 8, 0, 2) \
-   X(1, 64, 1, 0, 16) X(1, 64, 2, 0, 8) X(1, 64, 4, 0, 4) X(1, 64, 8, 0, 2)
+   X(4, 8, 1, 1, FMM_U(8)) X(4, 16, 1, 1, FMM_U(8)) X(4, 32, 1, 1, FMM_U(8)) X(4, 64, 1, 1, FMM_U(16)) \
+   X(4, 64, 2, 1, FMM_U(8)) \
+   X(4, 8, 1, 0, FMM_U(8)) X(4, 16, 1, 0, FMM_U(8)) X(4, 32, 1, 0, FMM_U(8)) X(4, 64, 1, 0, FMM_U(16)) \
+   X(4, 64, 2, 0, FMM_U(8)) X(4, 64, 4, 0, FMM_U(4)) X(4, 64, 8, 0, FMM_U(2)) \
+   X(1, 64, 1, 0, FMM_U(16)) X(1, 64, 2, 0, FMM_U(8)) X(1, 64, 4, 0, FMM_U(4)) X(1, 64, 8, 0, FMM_U(2))
 
 struct Launch {
    int num_cu, blocks_per_cu;
@@ -292,12 +313,12 @@ int make_plan(int32_t imsg, int opt_enabled, Plan *pl)
 struct Args {
    int32_t imessage;
    int64_t m, n, k, nnz;
-   const float *val;
+   const val_t *val;
    const idx_t *indx, *pntrb, *pntre;
-   const float *x, *y;
-   float *z;
+   const val_t *x, *y;
+   val_t *z;
    int64_t ldx, ldy, ldz;
-   float beta;
+   val_t beta;
 };
 
 // Everything here is device memory.  Enqueues on `stream`, does not wait.
@@ -324,8 +345,10 @@ int run_on_device(const Args &a, const Plan &pl, int sop_kind, hipStream_t strea
    int st = device_state(&d);
    if (st) return st;
 
-   const bool vec_ok = (a.k % 4 == 0) && (a.ldy % 4 == 0) && (a.ldz % 4 == 0) && aligned16(a.y) && aligned16(a.z) &&
-                       (!pl.reads_x || ((a.ldx % 4 == 0) && aligned16(a.x)));
+   // 16-byte accesses need 16-byte aligned rows: leading dimensions a multiple of 4 floats / 2 doubles
+   constexpr int64_t ld_mult = 16 / (int64_t)kValBytes;
+   const bool vec_ok = (a.k % 4 == 0) && (a.ldy % ld_mult == 0) && (a.ldz % ld_mult == 0) && aligned16(a.y) &&
+                       aligned16(a.z) && (!pl.reads_x || ((a.ldx % ld_mult == 0) && aligned16(a.x)));
    Shape sh;
    st = pick_shape((int)a.k, vec_ok, &sh);
    if (st) return st;
@@ -343,7 +366,7 @@ int run_on_device(const Args &a, const Plan &pl, int sop_kind, hipStream_t strea
    p.sigmoid_table = d->sigmoid_table;
 
    // heavy-row split: segments of about 256 KiB of gathered rows
-   int seg_len = g.seg_len > 0 ? g.seg_len : (int)(262144 / (4 * a.k));
+   int seg_len = g.seg_len > 0 ? g.seg_len : (int)(262144 / ((int64_t)kValBytes * a.k));
    if (seg_len < 64 && g.seg_len <= 0) seg_len = 64;
    int64_t heavy_deg = g.heavy_deg > 0 ? g.heavy_deg : 2 * (int64_t)seg_len;
    if (heavy_deg < seg_len) heavy_deg = seg_len;
@@ -358,16 +381,16 @@ int run_on_device(const Args &a, const Plan &pl, int sop_kind, hipStream_t strea
    int64_t cap_seg = nnz_hint / seg_len * 3 / 2 + 1024;   // a row of d edges has at most d/seg_len + 1 segments
    int64_t cap_heavy = nnz_hint / heavy_deg + 1024;
    const int64_t max_partial_bytes = (int64_t)8 << 30;
-   if (cap_seg * p.kpad * 4 > max_partial_bytes) cap_seg = max_partial_bytes / (p.kpad * 4);
+   if (cap_seg * p.kpad * (int64_t)kValBytes > max_partial_bytes) cap_seg = max_partial_bytes / (p.kpad * (int64_t)kValBytes);
    if (cap_seg > 0x7FFFFFFF) cap_seg = 0x7FFFFFFF;
    if (cap_heavy > 0x7FFFFFFF) cap_heavy = 0x7FFFFFFF;
    st = grow(d->heavy, (size_t)cap_heavy * sizeof(HeavyRow)); if (st) return st;
    st = grow(d->segs, (size_t)cap_seg * sizeof(SegDesc)); if (st) return st;
-   st = grow(d->partial, (size_t)cap_seg * p.kpad * sizeof(float)); if (st) return st;
+   st = grow(d->partial, (size_t)cap_seg * p.kpad * kValBytes); if (st) return st;
    p.ctr = d->ctr;
    p.heavy = (HeavyRow *)d->heavy.ptr;
    p.segs = (SegDesc *)d->segs.ptr;
-   p.partial = (float *)d->partial.ptr;
+   p.partial = (val_t *)d->partial.ptr;
    p.cap_heavy = (unsigned int)cap_heavy;
    p.cap_seg = (unsigned int)cap_seg;
 
@@ -433,10 +456,10 @@ int stage_up(const Args &h, const Plan &pl, Args *a, int64_t *slots_out)
    if (need_val && !h.val) { FMM_LOG("NULL operand"); return FUSEDMM_FAIL_RETURN; }
    const size_t b_ptr = (size_t)h.m * sizeof(idx_t);
    const size_t b_idx = (size_t)(slots > 0 ? slots : 1) * sizeof(idx_t);
-   const size_t b_val = (size_t)(slots > 0 ? slots : 1) * sizeof(float);
-   const size_t b_x = (size_t)h.m * (size_t)h.ldx * sizeof(float);
-   const size_t b_y = (size_t)h.n * (size_t)h.ldy * sizeof(float);
-   const size_t b_z = (size_t)h.m * (size_t)h.ldz * sizeof(float);
+   const size_t b_val = (size_t)(slots > 0 ? slots : 1) * kValBytes;
+   const size_t b_x = (size_t)h.m * (size_t)h.ldx * kValBytes;
+   const size_t b_y = (size_t)h.n * (size_t)h.ldy * kValBytes;
+   const size_t b_z = (size_t)h.m * (size_t)h.ldz * kValBytes;
    st = grow(d->stage[0], b_ptr); if (st) return st;
    st = grow(d->stage[1], b_ptr); if (st) return st;
    st = grow(d->stage[2], b_idx); if (st) return st;
@@ -449,21 +472,21 @@ int stage_up(const Args &h, const Plan &pl, Args *a, int64_t *slots_out)
    FMM_HIP(hipMemcpyAsync(d->stage[0].ptr, h.pntrb, b_ptr, hipMemcpyHostToDevice, s));
    FMM_HIP(hipMemcpyAsync(d->stage[1].ptr, h.pntre, b_ptr, hipMemcpyHostToDevice, s));
    if (slots > 0) FMM_HIP(hipMemcpyAsync(d->stage[2].ptr, h.indx, (size_t)slots * sizeof(idx_t), hipMemcpyHostToDevice, s));
-   if (need_val && slots > 0) FMM_HIP(hipMemcpyAsync(d->stage[3].ptr, h.val, (size_t)slots * sizeof(float), hipMemcpyHostToDevice, s));
+   if (need_val && slots > 0) FMM_HIP(hipMemcpyAsync(d->stage[3].ptr, h.val, (size_t)slots * kValBytes, hipMemcpyHostToDevice, s));
    if (pl.reads_x) FMM_HIP(hipMemcpyAsync(d->stage[4].ptr, h.x, b_x, hipMemcpyHostToDevice, s));
    FMM_HIP(hipMemcpyAsync(d->stage[5].ptr, h.y, b_y, hipMemcpyHostToDevice, s));
    const bool overwrite = pl.opt_rule && h.beta == 0.0f;
    if (!overwrite)
-      FMM_HIP(hipMemcpy2DAsync(d->stage[6].ptr, (size_t)h.ldz * 4, h.z, (size_t)h.ldz * 4, (size_t)h.k * 4, (size_t)h.m,
+      FMM_HIP(hipMemcpy2DAsync(d->stage[6].ptr, (size_t)h.ldz * kValBytes, h.z, (size_t)h.ldz * kValBytes, (size_t)h.k * kValBytes, (size_t)h.m,
                                hipMemcpyHostToDevice, s));
    *a = h;
    a->pntrb = (const idx_t *)d->stage[0].ptr;
    a->pntre = (const idx_t *)d->stage[1].ptr;
    a->indx = (const idx_t *)d->stage[2].ptr;
-   a->val = need_val ? (const float *)d->stage[3].ptr : nullptr;
-   a->x = pl.reads_x ? (const float *)d->stage[4].ptr : nullptr;
-   a->y = (const float *)d->stage[5].ptr;
-   a->z = (float *)d->stage[6].ptr;
+   a->val = need_val ? (const val_t *)d->stage[3].ptr : nullptr;
+   a->x = pl.reads_x ? (const val_t *)d->stage[4].ptr : nullptr;
+   a->y = (const val_t *)d->stage[5].ptr;
+   a->z = (val_t *)d->stage[6].ptr;
    if (a->nnz <= 0 || a->nnz > slots) a->nnz = slots;
    *slots_out = slots;
    return FUSEDMM_SUCCESS_RETURN;
@@ -473,7 +496,7 @@ int stage_up(const Args &h, const Plan &pl, Args *a, int64_t *slots_out)
 // touches nothing else.
 int stage_down(const Args &h, const Args &a)
 {
-   FMM_HIP(hipMemcpy2DAsync(h.z, (size_t)h.ldz * 4, a.z, (size_t)h.ldz * 4, (size_t)h.k * 4, (size_t)h.m,
+   FMM_HIP(hipMemcpy2DAsync(h.z, (size_t)h.ldz * kValBytes, a.z, (size_t)h.ldz * kValBytes, (size_t)h.k * kValBytes, (size_t)h.m,
                             hipMemcpyDeviceToHost, 0));
    FMM_HIP(hipStreamSynchronize(0));
    return FUSEDMM_SUCCESS_RETURN;
@@ -499,7 +522,7 @@ int run_staged(const Args &h, const Plan &pl, int sop_kind)
 // scalars as edge values.  Synchronous; device operands `a`, host copies of
 // the row pointers in h_pb / h_pe.
 template <int V, int L, int R, bool EXACT, int U>
-int launch_edge_scalar(const Params<idx_t> &p, float *s_out, int num_cu)
+int launch_edge_scalar(const Params<idx_t> &p, val_t *s_out, int num_cu)
 {
    int64_t blocks = (p.m + kWavesPerBlock - 1) / kWavesPerBlock;
    if (blocks > (int64_t)num_cu * 8) blocks = (int64_t)num_cu * 8;
@@ -519,14 +542,15 @@ int run_host_sop(const Args &a, const idx_t *h_pb, const idx_t *h_pe, int64_t sl
    const int vsc = GET_VSC_FLAG(a.imessage);
    const bool overwrite = pl.opt_rule && a.beta == 0.0f;
    if (overwrite)
-      FMM_HIP(hipMemset2DAsync(a.z, (size_t)a.ldz * 4, 0, (size_t)a.k * 4, (size_t)a.m, 0));
+      FMM_HIP(hipMemset2DAsync(a.z, (size_t)a.ldz * kValBytes, 0, (size_t)a.k * kValBytes, (size_t)a.m, 0));
    if (slots <= 0) return hip_status(hipStreamSynchronize(0), "hipStreamSynchronize");
-   st = grow(d->stage[7], (size_t)slots * sizeof(float));
+   st = grow(d->stage[7], (size_t)slots * kValBytes);
    if (st) return st;
-   float *d_s = (float *)d->stage[7].ptr;
+   val_t *d_s = (val_t *)d->stage[7].ptr;
 
    // pass 1
-   const bool vec_ok = (a.k % 4 == 0) && (a.ldy % 4 == 0) && aligned16(a.y) && (a.ldx % 4 == 0) && aligned16(a.x);
+   constexpr int64_t ld_mult = 16 / (int64_t)kValBytes;
+   const bool vec_ok = (a.k % 4 == 0) && (a.ldy % ld_mult == 0) && aligned16(a.y) && (a.ldx % ld_mult == 0) && aligned16(a.x);
    Shape sh;
    st = pick_shape((int)a.k, vec_ok, &sh);
    if (st) return st;
@@ -541,8 +565,8 @@ int run_host_sop(const Args &a, const idx_t *h_pb, const idx_t *h_pe, int64_t sl
    FMM_SHAPES(FMM_CASE)
 #undef FMM_CASE
    if (st) return st;
-   std::vector<float> hs((size_t)slots);
-   FMM_HIP(hipMemcpyAsync(hs.data(), d_s, (size_t)slots * sizeof(float), hipMemcpyDeviceToHost, 0));
+   std::vector<val_t> hs((size_t)slots);
+   FMM_HIP(hipMemcpyAsync(hs.data(), d_s, (size_t)slots * kValBytes, hipMemcpyDeviceToHost, 0));
    FMM_HIP(hipStreamSynchronize(0));
 
    // host SOP, rows dealt to a few threads (the function must be thread-safe, reference fusedMM.h:125-126)
@@ -557,13 +581,13 @@ int run_host_sop(const Args &a, const idx_t *h_pb, const idx_t *h_pe, int64_t sl
          for (int64_t i = lo; i < hi; i++)
             for (int64_t j = (int64_t)h_pb[i]; j < (int64_t)h_pe[i]; j++)
             {
-               float out = hs[(size_t)j];
+               val_t out = hs[(size_t)j];
                (void)fn(hs[(size_t)j], &out);
                hs[(size_t)j] = out;
             }
       });
    for (auto &th : pool) th.join();
-   FMM_HIP(hipMemcpyAsync(d_s, hs.data(), (size_t)slots * sizeof(float), hipMemcpyHostToDevice, 0));
+   FMM_HIP(hipMemcpyAsync(d_s, hs.data(), (size_t)slots * kValBytes, hipMemcpyHostToDevice, 0));
 
    // pass 2: same VOP / MOP / AOP, the scalar comes in as the edge value
    Args a2 = a;
@@ -667,11 +691,16 @@ int fusedMM_csr_stream(const int32_t imessage, const INDEXTYPE m, const INDEXTYP
    return entry(a, true, (hipStream_t)stream);
 }
 
-void sgfusedMM_csr(const char tkern, const INDEXTYPE m, const INDEXTYPE n, const INDEXTYPE k, const float alpha,
-                   const INDEXTYPE nnz, const INDEXTYPE rows, const INDEXTYPE cols, const float *val,
-                   const INDEXTYPE *indx, const INDEXTYPE *pntrb, const INDEXTYPE *pntre, const float *a,
-                   const INDEXTYPE lda, const float *b, const INDEXTYPE ldb, const float beta, float *c,
-                   const INDEXTYPE ldc)
+#ifdef FMM_DOUBLE
+#define FMM_GFUSEDMM dgfusedMM_csr
+#else
+#define FMM_GFUSEDMM sgfusedMM_csr
+#endif
+void FMM_GFUSEDMM(const char tkern, const INDEXTYPE m, const INDEXTYPE n, const INDEXTYPE k, const VALUETYPE alpha,
+                  const INDEXTYPE nnz, const INDEXTYPE rows, const INDEXTYPE cols, const VALUETYPE *val,
+                  const INDEXTYPE *indx, const INDEXTYPE *pntrb, const INDEXTYPE *pntre, const VALUETYPE *a,
+                  const INDEXTYPE lda, const VALUETYPE *b, const INDEXTYPE ldb, const VALUETYPE beta, VALUETYPE *c,
+                  const INDEXTYPE ldc)
 {
    int32_t imsg;
    switch (tkern)
@@ -688,6 +717,8 @@ void sgfusedMM_csr(const char tkern, const INDEXTYPE m, const INDEXTYPE n, const
 }
 
 int fusedMM_amd_index_bytes(void) { return (int)sizeof(INDEXTYPE); }
+
+int fusedMM_amd_value_bytes(void) { return (int)sizeof(VALUETYPE); }
 
 int fusedMM_amd_set_sop_kind(int kind)
 {

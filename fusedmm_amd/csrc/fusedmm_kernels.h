@@ -20,6 +20,16 @@
 
 namespace fmm {
 
+// The library is compiled once per value type, as the reference is (-DDREAL).
+#ifdef FMM_DOUBLE
+typedef double real_t;
+#else
+typedef float real_t;
+#endif
+struct alignas(16) real4 {
+   real_t x, y, z, w;
+};
+
 // ---- op-tuple nibbles (values of the public header) -------------------------
 enum : int {
    kVopCopyLhs = 0x1, kVopCopyRhs = 0x2, kVopAdd = 0x3, kVopSubl = 0x4, kVopSubr = 0x5,
@@ -73,39 +83,60 @@ constexpr unsigned int kMaxSegsPerRow = 512;   // longer rows get longer segment
 template <typename IdxT>
 struct Params {
    const IdxT *pntrb, *pntre, *indx;
-   const float *val;
-   const float *x, *y;
-   float *z;
+   const real_t *val;
+   const real_t *x, *y;
+   real_t *z;
    int64_t m;
    int64_t ldx, ldy, ldz;
    int k;
    int beta_zero;          // 1: overwrite Z, 0: accumulate into Z
    int sop_kind;           // device SOP body for SOP_UDEF
    int imessage;           // op tuple (read by OP_GENERIC only)
-   const float *sigmoid_table;
+   const real_t *sigmoid_table;
    // heavy-row queue
    int64_t heavy_deg;      // rows with more edges than this are split
    int seg_len;            // edges per segment
    Counters *ctr;
    HeavyRow *heavy;
    SegDesc *segs;
-   float *partial;         // [cap_seg][kpad]
+   real_t *partial;        // [cap_seg][kpad]
    unsigned int cap_heavy, cap_seg;
    int kpad;
    int row_counters;       // claim counters in use: kRowCounters, or 1 when the grid has fewer waves
 };
 
 // ---- wave primitives --------------------------------------------------------
+// Cross-lane moves work on 32-bit registers; a double is moved as two halves.
 __device__ __forceinline__ float as_f(int v) { return __builtin_bit_cast(float, v); }
 __device__ __forceinline__ int as_i(float v) { return __builtin_bit_cast(int, v); }
 
 template <int CTRL>
-__device__ __forceinline__ float dpp(float v)
+__device__ __forceinline__ int dpp_i(int v) { return __builtin_amdgcn_update_dpp(0, v, CTRL, 0xF, 0xF, false); }
+__device__ __forceinline__ int xor16_i(int v) { return __builtin_amdgcn_ds_swizzle(v, 0x401F); }
+
+#define FMM_SPLIT64(v, lo, hi)                                    \
+   const long long bits_ = __builtin_bit_cast(long long, v);      \
+   const int lo = (int)(bits_ & 0xFFFFFFFFll), hi = (int)(bits_ >> 32)
+__device__ __forceinline__ double join64(int lo, int hi)
 {
-   return as_f(__builtin_amdgcn_update_dpp(0, as_i(v), CTRL, 0xF, 0xF, false));
+   return __builtin_bit_cast(double, ((long long)hi << 32) | (long long)(unsigned int)lo);
 }
-// value held by lane ^ 16 / lane ^ 32
-__device__ __forceinline__ float lane_xor16(float v) { return as_f(__builtin_amdgcn_ds_swizzle(as_i(v), 0x401F)); }
+
+template <int CTRL>
+__device__ __forceinline__ float dpp(float v) { return as_f(dpp_i<CTRL>(as_i(v))); }
+template <int CTRL>
+__device__ __forceinline__ double dpp(double v)
+{
+   FMM_SPLIT64(v, lo, hi);
+   return join64(dpp_i<CTRL>(lo), dpp_i<CTRL>(hi));
+}
+// value held by lane ^ 16
+__device__ __forceinline__ float lane_xor16(float v) { return as_f(xor16_i(as_i(v))); }
+__device__ __forceinline__ double lane_xor16(double v)
+{
+   FMM_SPLIT64(v, lo, hi);
+   return join64(xor16_i(lo), xor16_i(hi));
+}
 
 // v[lane] + v[lane ^ 32]: one v_permlane32_swap gives both halves to every lane.
 __device__ __forceinline__ float add_xor32(float v)
@@ -113,12 +144,24 @@ __device__ __forceinline__ float add_xor32(float v)
    auto r = __builtin_amdgcn_permlane32_swap(as_i(v), as_i(v), false, false);
    return as_f(r[0]) + as_f(r[1]);
 }
+__device__ __forceinline__ double add_xor32(double v)
+{
+   FMM_SPLIT64(v, lo, hi);
+   auto a = __builtin_amdgcn_permlane32_swap(lo, lo, false, false);
+   auto b = __builtin_amdgcn_permlane32_swap(hi, hi, false, false);
+   return join64(a[0], b[0]) + join64(a[1], b[1]);
+}
+
+__device__ __forceinline__ float fma_r(float a, float b, float c) { return __builtin_fmaf(a, b, c); }
+__device__ __forceinline__ double fma_r(double a, double b, double c) { return __builtin_fma(a, b, c); }
+__device__ __forceinline__ real_t max_r(real_t a, real_t b) { return a > b ? a : b; }
+__device__ __forceinline__ real_t min_r(real_t a, real_t b) { return a < b ? a : b; }
 
 // Sum over the L lanes of a sub-wave; every lane ends with the same bits.
 // After the quad steps all lanes of a quad agree, so the half-row and row
 // mirrors deliver exactly the value lane^4 / lane^8 holds.
 template <int L>
-__device__ __forceinline__ float subwave_sum(float v)
+__device__ __forceinline__ real_t subwave_sum(real_t v)
 {
    if (L >= 2) v = v + dpp<0xB1>(v);   // quad_perm [1,0,3,2]  : lane ^ 1
    if (L >= 4) v = v + dpp<0x4E>(v);   // quad_perm [2,3,0,1]  : lane ^ 2
@@ -132,7 +175,7 @@ __device__ __forceinline__ float subwave_sum(float v)
 // Combine the S = 64/L sub-wave accumulators (same element slice, different
 // edges).  Offsets L, 2L .. 32 are true lane XORs (row_ror:8 == lane ^ 8).
 template <int L>
-__device__ __forceinline__ float cross_subwave_sum(float v)
+__device__ __forceinline__ real_t cross_subwave_sum(real_t v)
 {
    static_assert(L >= 8, "sub-waves narrower than 8 lanes are not used");
    if (L <= 8) v = v + dpp<0x128>(v);  // row_ror:8
@@ -141,19 +184,19 @@ __device__ __forceinline__ float cross_subwave_sum(float v)
    return v;
 }
 template <int L>
-__device__ __forceinline__ float cross_subwave_max(float v)
+__device__ __forceinline__ real_t cross_subwave_max(real_t v)
 {
-   if (L <= 8) v = fmaxf(v, dpp<0x128>(v));
-   if (L <= 16) v = fmaxf(v, lane_xor16(v));
-   if (L <= 32) v = fmaxf(v, __shfl_xor(v, 32, 64));
+   if (L <= 8) v = max_r(v, dpp<0x128>(v));
+   if (L <= 16) v = max_r(v, lane_xor16(v));
+   if (L <= 32) v = max_r(v, (real_t)__shfl_xor(v, 32, 64));
    return v;
 }
 template <int L>
-__device__ __forceinline__ float cross_subwave_min(float v)
+__device__ __forceinline__ real_t cross_subwave_min(real_t v)
 {
-   if (L <= 8) v = fminf(v, dpp<0x128>(v));
-   if (L <= 16) v = fminf(v, lane_xor16(v));
-   if (L <= 32) v = fminf(v, __shfl_xor(v, 32, 64));
+   if (L <= 8) v = min_r(v, dpp<0x128>(v));
+   if (L <= 16) v = min_r(v, lane_xor16(v));
+   if (L <= 32) v = min_r(v, (real_t)__shfl_xor(v, 32, 64));
    return v;
 }
 
@@ -185,8 +228,9 @@ __device__ __forceinline__ int64_t lane_value<int64_t>(int64_t v, int t)
 // ---- SOP bodies ---------------------------------------------------------------
 // Same expressions, in the same precision, as the SOP_UDEF_FUNC bodies of the
 // reference's tester (test/fusedMMtime.cpp:606-660): constants there are double
-// literals, so the arithmetic is done in double and rounded once to float.
-__device__ __forceinline__ float sop_eval(int kind, float s, const float *tab)
+// literals, so the arithmetic is done in double and (single-precision build)
+// rounded once to float.
+__device__ __forceinline__ real_t sop_eval(int kind, real_t s, const real_t *tab)
 {
    switch (kind)
    {
@@ -194,60 +238,89 @@ __device__ __forceinline__ float sop_eval(int kind, float s, const float *tab)
       {
          // floor-indexed 2048-entry table on [-5,5] (test/fusedMMtime.cpp:128-130, 606-611);
          // s == 5 exactly would index one past the end there: clamp to the last entry.
-         float t;
-         if (s > 5.0f) t = 1.0f;
-         else if (s < -5.0f) t = 0.0f;
+         real_t t;
+         if (s > (real_t)5.0) t = (real_t)1.0;
+         else if (s < (real_t)-5.0) t = (real_t)0.0;
          else
          {
+#ifdef FMM_DOUBLE
+            int idx = (int)((s + 5.0) * 2048.0 / 10.0);
+#else
             // The reference evaluates ((double)s + 5.0) * 2048 / 10.0.  One multiply by
             // 204.8 truncates to the same integer for every float in [-5, 5]
             // (checked exhaustively over all 2 168 455 170 of them on the CPU), and
             // spares a double-precision division per edge.
             int idx = (int)(((double)s + 5.0) * 204.8);
+#endif
             idx = idx > kSigmoidTableSize - 1 ? kSigmoidTableSize - 1 : idx;
             t = tab[idx];
          }
-         return 1.0f - t;   // exact in double for table values, so one rounding either way
+         return (real_t)1.0 - t;   // single precision: exact in double for table values, one rounding either way
       }
       case SOP_TDIST:
       {
-         float t = (float)(-2.0 / (1.0 + (double)s));
-         t = t > 5.0f ? 5.0f : t;
-         t = t < -5.0f ? -5.0f : t;
+         real_t t = (real_t)(-2.0 / (1.0 + (double)s));
+         t = t > (real_t)5.0 ? (real_t)5.0 : t;
+         t = t < (real_t)-5.0 ? (real_t)-5.0 : t;
          return t;
       }
       case SOP_FR:
-         return (float)(1.0 + 1.0 / (double)s);
+         return (real_t)(1.0 + 1.0 / (double)s);
+#ifdef FMM_DOUBLE
+      case SOP_LL:
+         return log2(1 + sqrt(s));
+      case SOP_FA:
+         return sqrt(s) + 1.0 / s;
+#else
       case SOP_LL:
          return log2f(1.0f + sqrtf(s));
       case SOP_FA:
          return (float)((double)sqrtf(s) + 1.0 / (double)s);
+#endif
       default:
          return s;
    }
 }
 
-__device__ __forceinline__ float4 ld4(const float *p) { return *reinterpret_cast<const float4 *>(p); }
-__device__ __forceinline__ void st4(float *p, float4 v) { *reinterpret_cast<float4 *>(p) = v; }
+// Four consecutive elements: 16 bytes in single precision (one 16-byte access),
+// 32 bytes in double precision (two 16-byte accesses; rows need 16-byte alignment only).
+__device__ __forceinline__ real4 ld4(const real_t *p) { return *reinterpret_cast<const real4 *>(p); }
+__device__ __forceinline__ void st4(real_t *p, real4 v) { *reinterpret_cast<real4 *>(p) = v; }
 // Streaming variants for data touched once per call (X rows, Z rows): the
 // non-temporal hint keeps them from displacing gathered Y rows in the caches.
-typedef float v4f_t __attribute__((ext_vector_type(4)));
-__device__ __forceinline__ float4 ld4_stream(const float *p)
+#ifdef FMM_DOUBLE
+typedef double vec16_t __attribute__((ext_vector_type(2)));
+__device__ __forceinline__ real4 ld4_stream(const real_t *p)
 {
-   const v4f_t v = __builtin_nontemporal_load(reinterpret_cast<const v4f_t *>(p));
-   return make_float4(v.x, v.y, v.z, v.w);
+   const vec16_t a = __builtin_nontemporal_load(reinterpret_cast<const vec16_t *>(p));
+   const vec16_t b = __builtin_nontemporal_load(reinterpret_cast<const vec16_t *>(p) + 1);
+   return real4{a.x, a.y, b.x, b.y};
 }
-__device__ __forceinline__ void st4_stream(float *p, float4 v)
+__device__ __forceinline__ void st4_stream(real_t *p, real4 v)
 {
-   v4f_t t = {v.x, v.y, v.z, v.w};
-   __builtin_nontemporal_store(t, reinterpret_cast<v4f_t *>(p));
+   vec16_t a = {v.x, v.y}, b = {v.z, v.w};
+   __builtin_nontemporal_store(a, reinterpret_cast<vec16_t *>(p));
+   __builtin_nontemporal_store(b, reinterpret_cast<vec16_t *>(p) + 1);
 }
-__device__ __forceinline__ float4 zero4() { return make_float4(0.f, 0.f, 0.f, 0.f); }
+#else
+typedef float vec16_t __attribute__((ext_vector_type(4)));
+__device__ __forceinline__ real4 ld4_stream(const real_t *p)
+{
+   const vec16_t v = __builtin_nontemporal_load(reinterpret_cast<const vec16_t *>(p));
+   return real4{v.x, v.y, v.z, v.w};
+}
+__device__ __forceinline__ void st4_stream(real_t *p, real4 v)
+{
+   vec16_t t = {v.x, v.y, v.z, v.w};
+   __builtin_nontemporal_store(t, reinterpret_cast<vec16_t *>(p));
+}
+#endif
+__device__ __forceinline__ real4 zero4() { return real4{(real_t)0, (real_t)0, (real_t)0, (real_t)0}; }
 
-// One row slice per lane: R float4 registers.
+// One row slice per lane: R real4 registers.
 template <int R>
 struct Slice {
-   float4 v[R];
+   real4 v[R];
 };
 
 // V == 4: lane sl holds elements 4*(r*L+sl) .. +3 in register r (16-byte accesses).
@@ -255,7 +328,7 @@ struct Slice {
 // multiple of 4, or an unaligned base): component c of register r holds
 // element (4r+c)*L + sl, loaded and stored 4 bytes at a time.
 template <int V, int L, int R, bool EXACT, bool STREAM = false>
-__device__ __forceinline__ void load_slice(Slice<R> &s, const float *row, int sl, int k)
+__device__ __forceinline__ void load_slice(Slice<R> &s, const real_t *row, int sl, int k)
 {
 #pragma unroll
    for (int r = 0; r < R; r++)
@@ -269,16 +342,16 @@ __device__ __forceinline__ void load_slice(Slice<R> &s, const float *row, int sl
       else
       {
          const int e0 = (4 * r) * L + sl;
-         s.v[r].x = (e0 < k) ? row[e0] : 0.0f;
-         s.v[r].y = (e0 + L < k) ? row[e0 + L] : 0.0f;
-         s.v[r].z = (e0 + 2 * L < k) ? row[e0 + 2 * L] : 0.0f;
-         s.v[r].w = (e0 + 3 * L < k) ? row[e0 + 3 * L] : 0.0f;
+         s.v[r].x = (e0 < k) ? row[e0] : (real_t)0;
+         s.v[r].y = (e0 + L < k) ? row[e0 + L] : (real_t)0;
+         s.v[r].z = (e0 + 2 * L < k) ? row[e0 + 2 * L] : (real_t)0;
+         s.v[r].w = (e0 + 3 * L < k) ? row[e0 + 3 * L] : (real_t)0;
       }
    }
 }
 
 template <int V, int L, int R, bool EXACT, bool STREAM = false>
-__device__ __forceinline__ void store_slice(float *row, const Slice<R> &s, int sl, int k)
+__device__ __forceinline__ void store_slice(real_t *row, const Slice<R> &s, int sl, int k)
 {
 #pragma unroll
    for (int r = 0; r < R; r++)
@@ -304,24 +377,24 @@ __device__ __forceinline__ void store_slice(float *row, const Slice<R> &s, int s
 }
 
 template <int L, int R>
-__device__ __forceinline__ float dot_slices(const Slice<R> &a, const Slice<R> &b)
+__device__ __forceinline__ real_t dot_slices(const Slice<R> &a, const Slice<R> &b)
 {
-   float p = 0.0f;
+   real_t p = (real_t)0;
 #pragma unroll
    for (int r = 0; r < R; r++)
    {
-      p = __builtin_fmaf(a.v[r].x, b.v[r].x, p);
-      p = __builtin_fmaf(a.v[r].y, b.v[r].y, p);
-      p = __builtin_fmaf(a.v[r].z, b.v[r].z, p);
-      p = __builtin_fmaf(a.v[r].w, b.v[r].w, p);
+      p = fma_r(a.v[r].x, b.v[r].x, p);
+      p = fma_r(a.v[r].y, b.v[r].y, p);
+      p = fma_r(a.v[r].z, b.v[r].z, p);
+      p = fma_r(a.v[r].w, b.v[r].w, p);
    }
    return subwave_sum<L>(p);
 }
 
 template <int L, int R>
-__device__ __forceinline__ float sum_slice(const Slice<R> &a)
+__device__ __forceinline__ real_t sum_slice(const Slice<R> &a)
 {
-   float p = 0.0f;
+   real_t p = (real_t)0;
 #pragma unroll
    for (int r = 0; r < R; r++) p = ((((p + a.v[r].x) + a.v[r].y) + a.v[r].z) + a.v[r].w);
    return subwave_sum<L>(p);
@@ -329,15 +402,15 @@ __device__ __forceinline__ float sum_slice(const Slice<R> &a)
 
 // acc = fma(d, t, acc) over a slice
 template <int R>
-__device__ __forceinline__ void axpy_slice(Slice<R> &acc, float d, const Slice<R> &t)
+__device__ __forceinline__ void axpy_slice(Slice<R> &acc, real_t d, const Slice<R> &t)
 {
 #pragma unroll
    for (int r = 0; r < R; r++)
    {
-      acc.v[r].x = __builtin_fmaf(d, t.v[r].x, acc.v[r].x);
-      acc.v[r].y = __builtin_fmaf(d, t.v[r].y, acc.v[r].y);
-      acc.v[r].z = __builtin_fmaf(d, t.v[r].z, acc.v[r].z);
-      acc.v[r].w = __builtin_fmaf(d, t.v[r].w, acc.v[r].w);
+      acc.v[r].x = fma_r(d, t.v[r].x, acc.v[r].x);
+      acc.v[r].y = fma_r(d, t.v[r].y, acc.v[r].y);
+      acc.v[r].z = fma_r(d, t.v[r].z, acc.v[r].z);
+      acc.v[r].w = fma_r(d, t.v[r].w, acc.v[r].w);
    }
 }
 
@@ -369,30 +442,30 @@ __device__ __forceinline__ void map2(Slice<R> &o, const Slice<R> &a, const Slice
 
 // Identity element of the accumulate stage (what a sub-wave that did not load
 // Z starts from).
-__device__ __forceinline__ float aop_identity(int aop)
+__device__ __forceinline__ real_t aop_identity(int aop)
 {
-   if (aop == kAopMax) return -__builtin_inff();
-   if (aop == kAopMin) return __builtin_inff();
-   return 0.0f;
+   if (aop == kAopMax) return -(real_t)__builtin_inf();
+   if (aop == kAopMin) return (real_t)__builtin_inf();
+   return (real_t)0;
 }
 
 // T = VOP(x, y) and s = ROP(x, T) of the general pipeline (reference
 // fusedMM.c:28-202, 721-725); s starts as the edge value (:717).
 template <int L, int R>
-__device__ __forceinline__ float vop_rop(Slice<R> &t, const Slice<R> &xs, const Slice<R> &ys, float edge_val, int vop,
+__device__ __forceinline__ real_t vop_rop(Slice<R> &t, const Slice<R> &xs, const Slice<R> &ys, real_t edge_val, int vop,
                                          int rop)
 {
    switch (vop)
    {
       case kVopCopyLhs: t = xs; break;
       case kVopCopyRhs: t = ys; break;
-      case kVopAdd: map2(t, xs, ys, [](float a, float b) { return a + b; }); break;
-      case kVopSubl: map2(t, xs, ys, [](float a, float b) { return -a + b; }); break;
-      case kVopSubr: map2(t, xs, ys, [](float a, float b) { return a - b; }); break;
-      case kVopMax: map2(t, xs, ys, [](float a, float b) { return a > b ? a : b; }); break;
-      default: map2(t, xs, ys, [](float a, float b) { return a < b ? a : b; }); break;
+      case kVopAdd: map2(t, xs, ys, [](real_t a, real_t b) { return a + b; }); break;
+      case kVopSubl: map2(t, xs, ys, [](real_t a, real_t b) { return -a + b; }); break;
+      case kVopSubr: map2(t, xs, ys, [](real_t a, real_t b) { return a - b; }); break;
+      case kVopMax: map2(t, xs, ys, [](real_t a, real_t b) { return a > b ? a : b; }); break;
+      default: map2(t, xs, ys, [](real_t a, real_t b) { return a < b ? a : b; }); break;
    }
-   float scal = edge_val;
+   real_t scal = edge_val;
    switch (rop)
    {
       case kRopDot: scal = dot_slices<L, R>(xs, t); break;
@@ -409,7 +482,7 @@ __device__ __forceinline__ float vop_rop(Slice<R> &t, const Slice<R> &xs, const 
 // acc = AOP(acc, T).  `xs` is the X[i] slice, `ys` the gathered Y[c] slice.
 template <int L, int R, int OP>
 __device__ __forceinline__ void edge_step(Slice<R> &acc, const Slice<R> &xs, const Slice<R> &ys,
-                                          float edge_val, int sop_kind, int imsg, const float *tab)
+                                          real_t edge_val, int sop_kind, int imsg, const real_t *tab)
 {
    if (OP == OP_GCN)
    {
@@ -428,16 +501,16 @@ __device__ __forceinline__ void edge_step(Slice<R> &acc, const Slice<R> &xs, con
    }
    else if (OP == OP_DOT)
    {
-      const float s = dot_slices<L, R>(xs, ys);
-      const float d = sop_eval(sop_kind, s, tab);
+      const real_t s = dot_slices<L, R>(xs, ys);
+      const real_t d = sop_eval(sop_kind, s, tab);
       axpy_slice<R>(acc, d, ys);
    }
    else if (OP == OP_DIST)
    {
       Slice<R> t;
       sub_slices<R>(t, xs, ys);
-      const float s = dot_slices<L, R>(t, t);
-      const float d = sop_eval(sop_kind, s, tab);
+      const real_t s = dot_slices<L, R>(t, t);
+      const real_t d = sop_eval(sop_kind, s, tab);
       axpy_slice<R>(acc, d, t);
    }
    else
@@ -445,8 +518,8 @@ __device__ __forceinline__ void edge_step(Slice<R> &acc, const Slice<R> &xs, con
       const int vop = imsg & 0xF, rop = imsg & 0xF0, sop = imsg & 0xF00, vsc = imsg & 0xF000,
                 aop = imsg & 0xF0000;
       Slice<R> t;
-      const float scal = vop_rop<L, R>(t, xs, ys, edge_val, vop, rop);
-      const float d = (sop == kSopUdef) ? sop_eval(sop_kind, scal, tab) : scal;
+      const real_t scal = vop_rop<L, R>(t, xs, ys, edge_val, vop, rop);
+      const real_t d = (sop == kSopUdef) ? sop_eval(sop_kind, scal, tab) : scal;
       if (vsc == kVscMul)
       {
 #pragma unroll
@@ -465,9 +538,9 @@ __device__ __forceinline__ void edge_step(Slice<R> &acc, const Slice<R> &xs, con
             t.v[r].z = d + t.v[r].z; t.v[r].w = d + t.v[r].w;
          }
       }
-      if (aop == kAopAdd) map2(acc, acc, t, [](float a, float b) { return a + b; });
-      else if (aop == kAopMax) map2(acc, acc, t, [](float a, float b) { return a > b ? a : b; });
-      else if (aop == kAopMin) map2(acc, acc, t, [](float a, float b) { return a < b ? a : b; });
+      if (aop == kAopAdd) map2(acc, acc, t, [](real_t a, real_t b) { return a + b; });
+      else if (aop == kAopMax) map2(acc, acc, t, [](real_t a, real_t b) { return a > b ? a : b; });
+      else if (aop == kAopMin) map2(acc, acc, t, [](real_t a, real_t b) { return a < b ? a : b; });
    }
 }
 
@@ -475,7 +548,7 @@ __device__ __forceinline__ void edge_step(Slice<R> &acc, const Slice<R> &xs, con
 template <typename IdxT>
 struct EdgeChunk {
    IdxT col;
-   float val;
+   real_t val;
 };
 
 template <int OP, typename IdxT>
@@ -483,7 +556,7 @@ __device__ __forceinline__ void load_chunk(EdgeChunk<IdxT> &c, const Params<IdxT
 {
    const IdxT j = j0 + lane;
    c.col = 0;
-   c.val = 0.0f;
+   c.val = (real_t)0;
    if (j < je)
    {
       c.col = p.indx[j];
@@ -512,6 +585,12 @@ __device__ __forceinline__ float chunk_entry(float v, int e)
 {
    return as_f(chunk_entry<L>(as_i(v), e));
 }
+template <int L>
+__device__ __forceinline__ double chunk_entry(double v, int e)
+{
+   FMM_SPLIT64(v, lo, hi);
+   return join64(chunk_entry<L>(lo, e), chunk_entry<L>(hi, e));
+}
 
 // Edges [jb, je) of one row, dealt round-robin to the sub-waves.  Column ids
 // (and edge values) are fetched 64 at a time with one coalesced load per
@@ -519,7 +598,7 @@ __device__ __forceinline__ float chunk_entry(float v, int e)
 // flight per sub-wave.  All lanes of the wave call this with the same jb, je.
 template <int V, int L, int R, bool EXACT, int OP, int SOPK, int U, typename IdxT>
 __device__ __forceinline__ void walk_edges(Slice<R> &acc, const Slice<R> &xs, const Params<IdxT> &p,
-                                           IdxT jb, IdxT je, int lane, const float *tab)
+                                           IdxT jb, IdxT je, int lane, const real_t *tab)
 {
    constexpr int S = 64 / L;
    const int sub = (L == 64) ? 0 : lane / L, sl = (L == 64) ? lane : lane % L;
@@ -531,13 +610,13 @@ __device__ __forceinline__ void walk_edges(Slice<R> &acc, const Slice<R> &xs, co
    {
       EdgeChunk<IdxT> nxt;
       nxt.col = 0;
-      nxt.val = 0.0f;
+      nxt.val = (real_t)0;
       if (j0 + 64 < je) load_chunk<OP, IdxT>(nxt, p, j0 + 64, je, lane);
       const int n = (je - j0) < 64 ? (int)(je - j0) : 64;
       for (int b0 = 0; b0 < n; b0 += S * U)
       {
          IdxT col[U];
-         float ev[U];
+         real_t ev[U];
          bool ok[U];
          Slice<R> ys[U];
 #pragma unroll
@@ -546,7 +625,7 @@ __device__ __forceinline__ void walk_edges(Slice<R> &acc, const Slice<R> &xs, co
             const int e = b0 + u * S + sub;     // L == 64: sub == 0, e is uniform
             ok[u] = e < n;
             col[u] = chunk_entry<L>(cur.col, e & 63);
-            ev[u] = (OP == OP_SPMM || OP == OP_GENERIC) ? chunk_entry<L>(cur.val, e & 63) : 0.0f;
+            ev[u] = (OP == OP_SPMM || OP == OP_GENERIC) ? chunk_entry<L>(cur.val, e & 63) : (real_t)0;
          }
 #pragma unroll
          for (int u = 0; u < U; u++)
@@ -597,7 +676,7 @@ __device__ __forceinline__ bool op_reads_x(int imsg)
    return false;
 }
 
-__device__ __forceinline__ const float *stage_table(const float *gtab, float *lds, bool need)
+__device__ __forceinline__ const real_t *stage_table(const real_t *gtab, real_t *lds, bool need)
 {
    if (!need) return gtab;
    for (int i = threadIdx.x; i < kSigmoidTableSize; i += kBlockThreads) lds[i] = gtab[i];
@@ -638,9 +717,9 @@ template <int V, int L, int R, bool EXACT, int OP, int SOPK, int U, typename Idx
 __global__ __launch_bounds__(kBlockThreads) void rows_kernel(const Params<IdxT> p)
 {
    constexpr int S = 64 / L;
-   __shared__ float lds_tab[(OP >= OP_DOT) ? kSigmoidTableSize : 1];
+   __shared__ real_t lds_tab[(OP >= OP_DOT) ? kSigmoidTableSize : 1];
    const bool uses_sop = (OP == OP_DOT || OP == OP_DIST || (OP == OP_GENERIC && (p.imessage & 0xF00) == kSopUdef));
-   const float *tab = stage_table(p.sigmoid_table, lds_tab, (OP >= OP_DOT) && uses_sop && (SOPK >= 0 ? SOPK : p.sop_kind) == SOP_SIGMOID);
+   const real_t *tab = stage_table(p.sigmoid_table, lds_tab, (OP >= OP_DOT) && uses_sop && (SOPK >= 0 ? SOPK : p.sop_kind) == SOP_SIGMOID);
 
    const int lane = threadIdx.x & 63;
    const int sub = lane / L, sl = lane % L;
@@ -719,7 +798,7 @@ __global__ __launch_bounds__(kBlockThreads) void rows_kernel(const Params<IdxT> 
 #pragma unroll
          for (int r = 0; r < R; r++) xs.v[r] = zero4();
       }
-      float *zrow = p.z + row * p.ldz;
+      real_t *zrow = p.z + row * p.ldz;
       if (generic)
       {
          // general semantics: fold the edges into the caller's Z with AOP
@@ -727,9 +806,9 @@ __global__ __launch_bounds__(kBlockThreads) void rows_kernel(const Params<IdxT> 
          if (sub == 0) load_slice<V, L, R, EXACT>(acc, zrow, sl, p.k);
          else
          {
-            const float id = aop_identity(aop);
+            const real_t id = aop_identity(aop);
 #pragma unroll
-            for (int r = 0; r < R; r++) acc.v[r] = make_float4(id, id, id, id);
+            for (int r = 0; r < R; r++) acc.v[r] = real4{id, id, id, id};
          }
       }
       else
@@ -747,7 +826,7 @@ __global__ __launch_bounds__(kBlockThreads) void rows_kernel(const Params<IdxT> 
          {
             Slice<R> zin;
             load_slice<V, L, R, EXACT>(zin, zrow, sl, p.k);
-            map2(acc, zin, acc, [](float a, float b) { return a + b; });
+            map2(acc, zin, acc, [](real_t a, real_t b) { return a + b; });
          }
          store_slice<V, L, R, EXACT, true>(zrow, acc, sl, p.k);
       }
@@ -760,12 +839,12 @@ __global__ __launch_bounds__(kBlockThreads) void rows_kernel(const Params<IdxT> 
 template <int V, int L, int R, bool EXACT, int OP, int SOPK, int U, typename IdxT>
 __global__ __launch_bounds__(kBlockThreads) void segments_kernel(const Params<IdxT> p)
 {
-   __shared__ float lds_tab[(OP >= OP_DOT) ? kSigmoidTableSize : 1];
+   __shared__ real_t lds_tab[(OP >= OP_DOT) ? kSigmoidTableSize : 1];
    unsigned int nseg = p.ctr->n_seg;
    if (nseg > p.cap_seg) nseg = p.cap_seg;   // rows beyond the cap were done inline
    if (nseg == 0) return;
    const bool uses_sop = (OP == OP_DOT || OP == OP_DIST || (OP == OP_GENERIC && (p.imessage & 0xF00) == kSopUdef));
-   const float *tab = stage_table(p.sigmoid_table, lds_tab, (OP >= OP_DOT) && uses_sop && (SOPK >= 0 ? SOPK : p.sop_kind) == SOP_SIGMOID);
+   const real_t *tab = stage_table(p.sigmoid_table, lds_tab, (OP >= OP_DOT) && uses_sop && (SOPK >= 0 ? SOPK : p.sop_kind) == SOP_SIGMOID);
 
    const int lane = threadIdx.x & 63;
    const int sub = lane / L, sl = lane % L;
@@ -794,9 +873,9 @@ __global__ __launch_bounds__(kBlockThreads) void segments_kernel(const Params<Id
 #pragma unroll
          for (int r = 0; r < R; r++) xs.v[r] = zero4();
       }
-      const float id = (OP == OP_GENERIC) ? aop_identity(aop) : 0.0f;
+      const real_t id = (OP == OP_GENERIC) ? aop_identity(aop) : (real_t)0;
 #pragma unroll
-      for (int r = 0; r < R; r++) acc.v[r] = make_float4(id, id, id, id);
+      for (int r = 0; r < R; r++) acc.v[r] = real4{id, id, id, id};
 
       walk_edges<V, L, R, EXACT, OP, SOPK, U, IdxT>(acc, xs, p, jb, je, lane, tab);
       merge_subwaves<L, R, OP>(acc, p.imessage);
@@ -813,7 +892,7 @@ __global__ __launch_bounds__(kBlockThreads) void segments_kernel(const Params<Id
 template <typename IdxT>
 __global__ __launch_bounds__(kBlockThreads) void merge_kernel(const Params<IdxT> p, int generic)
 {
-   __shared__ float red[kBlockThreads];
+   __shared__ real_t red[kBlockThreads];
    unsigned int nheavy = p.ctr->n_heavy;
    if (nheavy > p.cap_heavy) nheavy = p.cap_heavy;
    const int aop = p.imessage & 0xF0000;
@@ -826,14 +905,14 @@ __global__ __launch_bounds__(kBlockThreads) void merge_kernel(const Params<IdxT>
    {
       const HeavyRow hr = p.heavy[h];
       if (hr.n_seg == 0) continue;
-      float *zrow = p.z + hr.row * p.ldz;
+      real_t *zrow = p.z + hr.row * p.ldz;
       for (int e0 = 0; e0 < p.k; e0 += cols)
       {
          const int e = e0 + col;
          const bool live = active && e < p.k;
-         const float *pp = p.partial + (int64_t)hr.seg_base * p.kpad + e;
+         const real_t *pp = p.partial + (int64_t)hr.seg_base * p.kpad + e;
          const bool is_max = generic && aop == kAopMax, is_min = generic && aop == kAopMin;
-         float a = is_max ? -__builtin_inff() : (is_min ? __builtin_inff() : 0.0f);
+         real_t a = is_max ? -(real_t)__builtin_inf() : (is_min ? (real_t)__builtin_inf() : (real_t)0);
          if (live)
          {
             unsigned int s = grp;
@@ -841,15 +920,15 @@ __global__ __launch_bounds__(kBlockThreads) void merge_kernel(const Params<IdxT>
             {
                for (; s + 3u * G < hr.n_seg; s += 4u * G)
                {
-                  const float v0 = pp[(int64_t)s * p.kpad], v1 = pp[(int64_t)(s + G) * p.kpad],
+                  const real_t v0 = pp[(int64_t)s * p.kpad], v1 = pp[(int64_t)(s + G) * p.kpad],
                               v2 = pp[(int64_t)(s + 2u * G) * p.kpad], v3 = pp[(int64_t)(s + 3u * G) * p.kpad];
                   a += v0; a += v1; a += v2; a += v3;
                }
             }
             for (; s < hr.n_seg; s += G)
             {
-               const float v = pp[(int64_t)s * p.kpad];
-               a = is_max ? fmaxf(a, v) : (is_min ? fminf(a, v) : a + v);
+               const real_t v = pp[(int64_t)s * p.kpad];
+               a = is_max ? max_r(a, v) : (is_min ? min_r(a, v) : a + v);
             }
          }
          __syncthreads();
@@ -857,16 +936,16 @@ __global__ __launch_bounds__(kBlockThreads) void merge_kernel(const Params<IdxT>
          __syncthreads();
          if (live && grp == 0)
          {
-            float t = red[col];
+            real_t t = red[col];
             for (int g2 = 1; g2 < G; g2++)
             {
-               const float v = red[g2 * cols + col];
-               t = is_max ? fmaxf(t, v) : (is_min ? fminf(t, v) : t + v);
+               const real_t v = red[g2 * cols + col];
+               t = is_max ? max_r(t, v) : (is_min ? min_r(t, v) : t + v);
             }
             if (generic)
             {
-               const float zi = zrow[e];
-               t = is_max ? fmaxf(zi, t) : (is_min ? fminf(zi, t) : zi + t);
+               const real_t zi = zrow[e];
+               t = is_max ? max_r(zi, t) : (is_min ? min_r(zi, t) : zi + t);
             }
             else if (!p.beta_zero) t = zrow[e] + t;
             zrow[e] = t;
@@ -879,7 +958,7 @@ __global__ __launch_bounds__(kBlockThreads) void merge_kernel(const Params<IdxT>
 // One wave per row (static stride; this path exists for compatibility, the
 // host evaluates the caller's SOP_UDEF_FUNC on s[] before the accumulate pass).
 template <int V, int L, int R, bool EXACT, int U, typename IdxT>
-__global__ __launch_bounds__(kBlockThreads) void edge_scalar_kernel(const Params<IdxT> p, float *s_out)
+__global__ __launch_bounds__(kBlockThreads) void edge_scalar_kernel(const Params<IdxT> p, real_t *s_out)
 {
    constexpr int S = 64 / L;
    const int lane = threadIdx.x & 63;
@@ -903,7 +982,7 @@ __global__ __launch_bounds__(kBlockThreads) void edge_scalar_kernel(const Params
             {
                Slice<R> ys, t;
                load_slice<V, L, R, EXACT>(ys, p.y + (int64_t)p.indx[j] * p.ldy, sl, p.k);
-               const float scal = vop_rop<L, R>(t, xs, ys, p.val ? p.val[j] : 0.0f, vop, rop);
+               const real_t scal = vop_rop<L, R>(t, xs, ys, p.val ? p.val[j] : (real_t)0, vop, rop);
                if (sl == 0) s_out[j] = scal;
             }
          }

@@ -65,7 +65,8 @@ int fusedMM_csr_stream
 /*
  * The reference's second-level entry (kernels/include/kernels.h:32-37,
  * kernels/src/kernels.c:456-631): tkern 'g' gcn, 'm' spmm, 's' sigmoid,
- * 't' t-dist/FR.  Same pointer rules as fusedMM_csr.
+ * 't' t-dist/FR.  Same pointer rules as fusedMM_csr.  Exported by the
+ * single-precision libraries.
  */
 void sgfusedMM_csr
 (
@@ -76,8 +77,21 @@ void sgfusedMM_csr
    const float beta, float *c, const INDEXTYPE ldc
 );
 
-/* sizeof(INDEXTYPE) this library was built for (4 or 8). */
+/* The same for the double-precision libraries (kernels/include/kernels.h:17-22). */
+void dgfusedMM_csr
+(
+   const char tkern, const INDEXTYPE m, const INDEXTYPE n, const INDEXTYPE k,
+   const double alpha, const INDEXTYPE nnz, const INDEXTYPE rows, const INDEXTYPE cols,
+   const double *val, const INDEXTYPE *indx, const INDEXTYPE *pntrb, const INDEXTYPE *pntre,
+   const double *a, const INDEXTYPE lda, const double *b, const INDEXTYPE ldb,
+   const double beta, double *c, const INDEXTYPE ldc
+);
+
+/* sizeof(INDEXTYPE) and sizeof(VALUETYPE) this library was built for (4 or 8 each).
+ * Libraries: libfusedmm_amd_i32.so, _i64.so (float; the reference's default
+ * build) and libfusedmm_amd_d_i32.so, _d_i64.so (double; its -DDREAL build). */
 int fusedMM_amd_index_bytes(void);
+int fusedMM_amd_value_bytes(void);
 
 /* 1: pattern-matched tuples use the optimised kernels' write-back rule
  * (default, the reference's ENABLE_OPT_FUSEDMM build, fusedMM.c:512-605);

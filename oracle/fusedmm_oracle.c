@@ -58,147 +58,34 @@ enum {
    ORC_SOP_FA = 5        /* sqrt(val) + 1/val               (:656-660)  */
 };
 
-/* test/fusedMMtime.cpp:594-604 (uinit_SM_TABLE).  The harness is C++ and its
- * VALUETYPE is float, so `exp(-x)` resolves to the float overload and
- * `1 + exp(-x)` is a float sum; the quotient is formed in double and rounded
- * to float on assignment. */
-void orc_sigmoid_table(float *table)
-{
-   for (int i = 0; i < ORC_SM_TABLE_SIZE; i++)
-   {
-      float x = (float)(2.0 * ORC_SM_BOUND * i / ORC_SM_TABLE_SIZE - ORC_SM_BOUND);
-      float e = expf(-x);
-      float denom = 1 + e;
-      table[i] = (float)(1.0 / (double)denom);
-   }
-}
+/* ---- value-type dependent part, compiled for float and double ---- */
+#define ORC_VAL float
+#define ORC_VFN(name) name
+#define ORC_EXP expf
+#define ORC_SQRT sqrtf
+#define ORC_LOG2 log2f
+#define ORC_FMA fmaf
+#include "fusedmm_oracle_val.inc"
+#undef ORC_VAL
+#undef ORC_VFN
+#undef ORC_EXP
+#undef ORC_SQRT
+#undef ORC_LOG2
+#undef ORC_FMA
 
-/* Bin index of the floor-indexed lookup, test/fusedMMtime.cpp:128-130,606-611:
- * SM_RESOLUTION expands unparenthesised, so the expression is
- * ((double)v + 5.0) * 2048 / 10.0, truncated toward zero.  v == 5.0f would
- * index entry 2048 (one past the end in the reference); the restatement clamps
- * to 2047.  Returns -1 for v < -5 and 2048 for v > 5 (the saturated branches). */
-int orc_sigmoid_bin(float v)
-{
-   if (v > ORC_SM_BOUND) return ORC_SM_TABLE_SIZE;
-   if (v < -ORC_SM_BOUND) return -1;
-   int idx = (int)(((double)v + ORC_SM_BOUND) * ORC_SM_TABLE_SIZE / (2.0 * ORC_SM_BOUND));
-   if (idx > ORC_SM_TABLE_SIZE - 1) idx = ORC_SM_TABLE_SIZE - 1;
-   return idx;
-}
-
-/* test/fusedMMtime.cpp:606-611 (ufast_SM) */
-float orc_sigmoid_lookup(const float *table, float v)
-{
-   int b = orc_sigmoid_bin(v);
-   if (b >= ORC_SM_TABLE_SIZE) return 1.0f;
-   if (b < 0) return 0.0f;
-   return table[b];
-}
-
-static float g_table[ORC_SM_TABLE_SIZE];
-static int g_table_ready = 0;
-
-static const float *orc_table(void)
-{
-   if (!g_table_ready)
-   {
-#pragma omp critical(orc_table_init)
-      {
-         if (!g_table_ready)
-         {
-            orc_sigmoid_table(g_table);
-            g_table_ready = 1;
-         }
-      }
-   }
-   return g_table;
-}
-
-/* The harness's SOP_UDEF_FUNC bodies, test/fusedMMtime.cpp:626-674.  Constants
- * there are double literals, so each expression is evaluated in double and
- * rounded once to float on the store to *out; sqrt/log2 of a float argument
- * resolve to the float overloads in that C++ translation unit. */
-float orc_sop(int kind, float s)
-{
-   switch (kind)
-   {
-      case ORC_SOP_SIGMOID:
-         return (float)(1.0 - (double)orc_sigmoid_lookup(orc_table(), s));
-      case ORC_SOP_TDIST:
-      {
-         float t = (float)(-2.0 / (1.0 + (double)s)); /* tscale takes a float */
-         if (t > ORC_SM_BOUND) return (float)ORC_SM_BOUND;
-         if (t < -ORC_SM_BOUND) return (float)-ORC_SM_BOUND;
-         return t;
-      }
-      case ORC_SOP_FR:
-         return (float)(1.0 + 1.0 / (double)s);
-      case ORC_SOP_LL:
-      {
-         float r = 1 + sqrtf(s);
-         return log2f(r);
-      }
-      case ORC_SOP_FA:
-         return (float)((double)sqrtf(s) + 1.0 / (double)s);
-      default:
-         return s;
-   }
-}
-
-/* Vectorised form for the tests (fills out[i] = sop(kind, in[i])). */
-void orc_sop_array(int kind, const float *in, float *out, int64_t n)
-{
-   for (int64_t i = 0; i < n; i++) out[i] = orc_sop(kind, in[i]);
-}
-
-/*
- * Dot product (or squared distance) in the wavefront order the GPU kernels
- * use.  Not a restatement of reference code: it exists so that the table bin
- * chosen for an edge can be compared bit-for-bit between CPU and GPU, because
- * the reference's floor-indexed table makes the result discontinuous in the
- * dot (two summation orders can land in neighbouring bins).
- *
- * Element e of a K-vector lives in lane (e / V) % L, at position
- * (e / (V*L)) * V + e % V of that lane's private slice (V = floats per vector
- * load, L = lanes that share one row, a power of two).  Each lane forms a
- * fused-multiply-add chain over its slice in ascending position starting from
- * +0, then lanes are combined with an XOR butterfly, offsets 1, 2, 4 .. L/2,
- * each step p[l] = p[l] + p[l ^ off].
- *
- * diff == 0: sum x[e]*y[e].   diff == 1: sum (x[e]-y[e])^2.
- */
-float orc_gpu_dot(const float *x, const float *y, int64_t K, int V, int L, int diff)
-{
-   float p[64];
-   for (int l = 0; l < L; l++) p[l] = 0.0f;
-   int64_t nreg = (K + (int64_t)V * L - 1) / ((int64_t)V * L);
-   for (int l = 0; l < L; l++)
-   {
-      float acc = 0.0f;
-      for (int64_t r = 0; r < nreg; r++)
-         for (int c = 0; c < V; c++)
-         {
-            int64_t e = (r * L + l) * V + c;
-            if (e >= K) continue;
-            if (diff)
-            {
-               float t = x[e] - y[e];
-               acc = fmaf(t, t, acc);
-            }
-            else
-               acc = fmaf(x[e], y[e], acc);
-         }
-      p[l] = acc;
-   }
-   for (int off = 1; off < L; off <<= 1)
-   {
-      float q[64];
-      for (int l = 0; l < L; l++) q[l] = p[l] + p[l ^ off];
-      for (int l = 0; l < L; l++) p[l] = q[l];
-   }
-   return p[0];
-}
+#define ORC_VAL double
+#define ORC_VFN(name) name##_d
+#define ORC_EXP exp
+#define ORC_SQRT sqrt
+#define ORC_LOG2 log2
+#define ORC_FMA fma
+#include "fusedmm_oracle_val.inc"
+#undef ORC_VAL
+#undef ORC_VFN
+#undef ORC_EXP
+#undef ORC_SQRT
+#undef ORC_LOG2
+#undef ORC_FMA
 
 /* Counts the floats v in [-5, 5] for which the reference's bin expression
  * (orc_sigmoid_bin, a double division by 10.0) and the single multiply
@@ -232,15 +119,41 @@ int orc_max_threads(void)
 #endif
 }
 
-/* ---- index-width dependent part, compiled for int32_t and int64_t ---- */
+/* ---- index-width (and value-type) dependent part: four instances ---- */
+#define ORC_VAL float
+#define ORC_WIDE double
+#define ORC_VFN(name) name
+#define ORC_FMA fmaf
 #define ORC_IDX int32_t
 #define ORC_FN(name) name##_i32
 #include "fusedmm_oracle_body.inc"
 #undef ORC_IDX
 #undef ORC_FN
-
 #define ORC_IDX int64_t
 #define ORC_FN(name) name##_i64
 #include "fusedmm_oracle_body.inc"
 #undef ORC_IDX
 #undef ORC_FN
+#undef ORC_VAL
+#undef ORC_WIDE
+#undef ORC_VFN
+#undef ORC_FMA
+
+#define ORC_VAL double
+#define ORC_WIDE long double
+#define ORC_VFN(name) name##_d
+#define ORC_FMA fma
+#define ORC_IDX int32_t
+#define ORC_FN(name) name##_d_i32
+#include "fusedmm_oracle_body.inc"
+#undef ORC_IDX
+#undef ORC_FN
+#define ORC_IDX int64_t
+#define ORC_FN(name) name##_d_i64
+#include "fusedmm_oracle_body.inc"
+#undef ORC_IDX
+#undef ORC_FN
+#undef ORC_VAL
+#undef ORC_WIDE
+#undef ORC_VFN
+#undef ORC_FMA

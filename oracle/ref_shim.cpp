@@ -9,8 +9,8 @@
  *   fusedMM.c             (generic fusedMM_csr, :487-744, built the way the
  *                          reference builds its non-"Opt" executables)
  * The reference's optimised kernels need its code generator's output and are
- * therefore not part of this build.  One library per (SOP body, index width),
- * like the reference's one executable per kind.
+ * therefore not part of this build.  One library per (SOP body, precision,
+ * index width), like the reference's one executable per kind.
  *
  * This file contains no reference code: it only declares the reference's
  * symbols and forwards to them.
@@ -26,7 +26,11 @@
 #ifndef INDEXTYPE
 #error "build with -DINDEXTYPE=int32_t or int64_t"
 #endif
+#ifdef DREAL   /* the reference's switch for double precision */
+#define VALUETYPE double
+#else
 #define VALUETYPE float
+#endif
 
 #define REF_CSR_ARGS                                                                   \
    const char tkern, const INDEXTYPE m, const INDEXTYPE n, const INDEXTYPE k,          \
@@ -60,6 +64,7 @@ static CSR<INDEXTYPE, VALUETYPE> *g_csr = nullptr;
 extern "C" {
 
 int ref_index_bytes(void) { return (int)sizeof(INDEXTYPE); }
+int ref_value_bytes(void) { return (int)sizeof(VALUETYPE); }
 
 /* the harness's trusted kernel for tkern in {t,s,m,g,f} */
 void ref_trusted_csr(REF_CSR_ARGS) { mytrusted_csr(REF_CSR_PASS); }
@@ -82,14 +87,14 @@ int ref_fusedMM_csr(const int32_t imessage, const INDEXTYPE m, const INDEXTYPE n
 }
 
 /* the 2048-entry table exactly as the harness builds it */
-void ref_sm_table(float *out)
+void ref_sm_table(VALUETYPE *out)
 {
    if (!SM_TABLE) uinit_SM_TABLE();
-   std::memcpy(out, SM_TABLE, sizeof(float) * 2048);
+   std::memcpy(out, SM_TABLE, sizeof(VALUETYPE) * 2048);
 }
 
 /* the SOP_UDEF_FUNC body this library was compiled with */
-void ref_sop_array(const float *in, float *out, int64_t n)
+void ref_sop_array(const VALUETYPE *in, VALUETYPE *out, int64_t n)
 {
    if (!SM_TABLE) uinit_SM_TABLE();
    for (int64_t i = 0; i < n; i++) SOP_UDEF_FUNC(in[i], &out[i]);
@@ -111,12 +116,12 @@ int ref_load_mtx(const char *path, int64_t *rows, int64_t *cols, int64_t *nnz)
    return 0;
 }
 
-void ref_get_csr(INDEXTYPE *rowptr, INDEXTYPE *colids, float *values)
+void ref_get_csr(INDEXTYPE *rowptr, INDEXTYPE *colids, VALUETYPE *values)
 {
    if (!g_csr) return;
    std::memcpy(rowptr, g_csr->rowptr, sizeof(INDEXTYPE) * (size_t)(g_csr->rows + 1));
    std::memcpy(colids, g_csr->colids, sizeof(INDEXTYPE) * (size_t)g_csr->nnz);
-   std::memcpy(values, g_csr->values, sizeof(float) * (size_t)g_csr->nnz);
+   std::memcpy(values, g_csr->values, sizeof(VALUETYPE) * (size_t)g_csr->nnz);
 }
 
 } /* extern "C" */

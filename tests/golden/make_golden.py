@@ -6,7 +6,9 @@
 Fixtures are data only: inputs (small seeded graphs and embeddings, stored in
 full so nothing has to be regenerated bit-for-bit) and the reference's outputs:
   sop.npz             the harness's 2048-entry sigmoid table and its
-                      SOP_UDEF_FUNC bodies evaluated on a fixed probe vector
+                      SOP_UDEF_FUNC bodies evaluated on a fixed probe vector,
+                      single precision and (keys ending in _d) double precision
+  ops_d_i<bits>.npz   as ops_i<bits>.npz for the reference's -DDREAL build
   ops_i<bits>.npz     Z of the harness's trusted kernels and of the reference's
                       fusedMM_csr (general pipeline) for the five op kinds
   tuples_i32.npz      Z of the reference's fusedMM_csr for a sweep of op tuples
@@ -55,7 +57,34 @@ def main():
     for kind in ("sigmoid", "tdist", "fr", "ll", "fa"):
         arg = v if kind == "sigmoid" else np.abs(v) + np.float32(1e-3)
         out["sop_" + kind] = Ref(kind, 32).sop(arg)
+    vd = v.astype(np.float64)
+    vd = vd[vd < 4.99999]          # next to +5 the double build rounds v + 5 to 10 and reads past its table
+    out["probe_d"] = vd
+    out["table_d"] = Ref("sigmoid", 32, 64).table()
+    for kind in ("sigmoid", "tdist", "fr", "ll", "fa"):
+        arg = vd if kind == "sigmoid" else np.abs(vd) + 1e-3
+        out["sop_%s_d" % kind] = Ref(kind, 32, 64).sop(arg)
     np.savez_compressed(os.path.join(HERE, "sop.npz"), **out)
+
+    for bits in (32, 64):
+        out = {}
+        g = graphs.ragged(bits)
+        out["ragged_pntrb"], out["ragged_pntre"] = g["pntrb"], g["pntre"]
+        out["ragged_indx"], out["ragged_val"] = g["indx"], g["val"]
+        out["ragged_shape"] = np.array([g["rows"], g["cols"]])
+        k = 24
+        X = graphs.features(g["rows"], k, 1, -1, 1, 1).astype(np.float64)
+        Y = graphs.features(g["cols"], k, 1, -1, 1, 2).astype(np.float64)
+        out["ragged_X%d" % k], out["ragged_Y%d" % k] = X, Y
+        for t, kind in KINDS.items():
+            r = Ref(kind, bits, 64)
+            Zt = np.zeros((g["rows"], k))
+            r.trusted(t, g, X, Y, Zt)
+            Zf = np.zeros((g["rows"], k))
+            r.test(t, g, X, Y, Zf)
+            out["ragged_%s_k%d_trusted" % (t, k)] = Zt
+            out["ragged_%s_k%d_fusedmm" % (t, k)] = Zf
+        np.savez_compressed(os.path.join(HERE, "ops_d_i%d.npz" % bits), **out)
 
     for bits in (32, 64):
         out = {}

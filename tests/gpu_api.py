@@ -27,14 +27,14 @@ def layout_for(k, vec_ok=True):
 MAX_SEGS_PER_ROW = 512   # kMaxSegsPerRow of the kernels: longer rows get longer segments
 
 
-def default_split(k):
+def default_split(k, vbits=32):
     """(heavy_deg, seg_len) defaults of the library for feature width k."""
-    seg = max(64, 262144 // (4 * k))
+    seg = max(64, 262144 // ((vbits // 8) * k))
     return 2 * seg, seg
 
 
 def run(imsg, g, X, Y, Z, beta=0.0, bits=32, where="device", m=None, k=None, ldx=None, ldy=None, ldz=None,
-        nnz=None):
+        nnz=None, vbits=32):
     """Call fusedMM_csr.  where='device': operands copied to the GPU with torch
     and passed as device addresses; 'host': numpy arrays passed as they are.
     Returns (status, Z as numpy)."""
@@ -44,31 +44,34 @@ def run(imsg, g, X, Y, Z, beta=0.0, bits=32, where="device", m=None, k=None, ldx
     ldy = Y.shape[1] if ldy is None else ldy
     ldz = Z.shape[1] if ldz is None else ldz
     nnz = g["nnz"] if nnz is None else nnz
+    np_v = np.float32 if vbits == 32 else np.float64
+    gval = g["val"] if g["val"] is None or g["val"].dtype == np_v else g["val"].astype(np_v)
+    assert Y.dtype == np_v and Z.dtype == np_v and (X is None or X.dtype == np_v)
     if where == "host":
         Zh = np.ascontiguousarray(Z).copy()
-        rc = fa.fusedMM_csr(imsg, m, g["cols"], k, 1.0, nnz, g["rows"], g["cols"], g["val"], g["indx"],
+        rc = fa.fusedMM_csr(imsg, m, g["cols"], k, 1.0, nnz, g["rows"], g["cols"], gval, g["indx"],
                             np.ascontiguousarray(g["pntrb"]), np.ascontiguousarray(g["pntre"]),
-                            X, ldx, Y, ldy, beta, Zh, ldz, index_bits=bits)
+                            X, ldx, Y, ldy, beta, Zh, ldz, index_bits=bits, value_bits=vbits)
         return rc, Zh
     import torch
     dev = torch.device("cuda:0")
     t = lambda a: None if a is None else torch.from_numpy(np.ascontiguousarray(a)).to(dev)
-    val, indx, pb, pe = t(g["val"]), t(g["indx"]), t(g["pntrb"]), t(g["pntre"])
+    val, indx, pb, pe = t(gval), t(g["indx"]), t(g["pntrb"]), t(g["pntre"])
     Xd, Yd, Zd = t(X), t(Y), t(Z)
     rc = fa.fusedMM_csr(imsg, m, g["cols"], k, 1.0, nnz, g["rows"], g["cols"], val, indx, pb, pe,
-                        Xd, ldx, Yd, ldy, beta, Zd, ldz, index_bits=bits)
+                        Xd, ldx, Yd, ldy, beta, Zd, ldz, index_bits=bits, value_bits=vbits)
     torch.cuda.synchronize()
     return rc, Zd.cpu().numpy()
 
 
-def set_kind(kind, bits=32):
-    return fa.load(bits).fusedMM_amd_set_sop_kind(kind)
+def set_kind(kind, bits=32, vbits=32):
+    return fa.load(bits, vbits).fusedMM_amd_set_sop_kind(kind)
 
 
-def last_split(bits=32):
+def last_split(bits=32, vbits=32):
     import ctypes as C
     h, s, o = C.c_uint(), C.c_uint(), C.c_uint()
-    rc = fa.load(bits).fusedMM_amd_last_split(C.byref(h), C.byref(s), C.byref(o))
+    rc = fa.load(bits, vbits).fusedMM_amd_last_split(C.byref(h), C.byref(s), C.byref(o))
     assert rc == 0
     return h.value, s.value, o.value
 
@@ -100,7 +103,8 @@ def oracle_mirror(oracle, tkern, g, X, Y, Z0, beta, sop_kind, k, heavy_deg, seg_
     g2 = dict(g)
     g2.update(rows=len(pb), pntrb=np.array(pb, it), pntre=np.array(pe, it))
     X2 = None if X is None else np.ascontiguousarray(X[np.array(owner)])
-    P = np.zeros((len(pb), k), np.float32)
+    np_v = Z0.dtype.type
+    P = np.zeros((len(pb), k), np_v)
     oracle.opt(ot, g2, X2, Y, P, beta=0.0, sop_kind=sop_kind, mode=2, V=V, L=L, S=S)
     owner = np.array(owner)
     G = max(1, 256 // min(k, 256))          # merge kernel: groups of a 256-thread block
@@ -108,13 +112,13 @@ def oracle_mirror(oracle, tkern, g, X, Y, Z0, beta, sop_kind, k, heavy_deg, seg_
         mine = np.nonzero(owner == r)[0]
         total = None
         for grp in range(G):
-            a = np.zeros(k, np.float32)
+            a = np.zeros(k, np_v)
             for q in mine[grp::G]:
-                a = (a + P[q]).astype(np.float32)
-            total = a if total is None else (total + a).astype(np.float32)
-        Z[r] = total if beta == 0.0 else (Z0[r] + total).astype(np.float32)
+                a = (a + P[q]).astype(np_v)
+            total = a if total is None else (total + a).astype(np_v)
+        Z[r] = total if beta == 0.0 else (Z0[r] + total).astype(np_v)
     return Z
 
 
-def set_split(heavy_deg, seg_len, bits=32):
-    fa.load(bits).fusedMM_amd_set_split(heavy_deg, seg_len)
+def set_split(heavy_deg, seg_len, bits=32, vbits=32):
+    fa.load(bits, vbits).fusedMM_amd_set_split(heavy_deg, seg_len)

@@ -27,6 +27,10 @@ MSG = {
 _f32p = C.POINTER(C.c_float)
 
 
+def _vtype(vbits):
+    return (np.float32, C.c_float) if vbits == 32 else (np.float64, C.c_double)
+
+
 def _ptr(a, ctype):
     if a is None:
         return None
@@ -49,42 +53,54 @@ def _load(name):
 
 
 class Oracle:
-    """The CPU restatement.  fast=True loads the -O3 build (baseline timing)."""
+    """The CPU restatement.  fast=True loads the -O3 build (baseline timing);
+    vbits=64 selects the double-precision instance (the reference's -DDREAL)."""
 
-    def __init__(self, fast=False):
+    def __init__(self, fast=False, vbits=32):
         self.lib = _load("libfusedmm_oracle_fast.so" if fast else "libfusedmm_oracle.so")
+        self.vbits = vbits
+        self.np_v, self.cv = _vtype(vbits)
+        self.sfx = "" if vbits == 32 else "_d"
         L = self.lib
-        L.orc_sigmoid_table.argtypes = [_f32p]
-        L.orc_sigmoid_bin.argtypes = [C.c_float]
-        L.orc_sigmoid_bin.restype = C.c_int
-        L.orc_sop.argtypes = [C.c_int, C.c_float]
-        L.orc_sop.restype = C.c_float
-        L.orc_sop_array.argtypes = [C.c_int, _f32p, _f32p, C.c_int64]
-        L.orc_gpu_dot.argtypes = [_f32p, _f32p, C.c_int64, C.c_int, C.c_int, C.c_int]
-        L.orc_gpu_dot.restype = C.c_float
+        vp = C.POINTER(self.cv)
+        self._table = getattr(L, "orc_sigmoid_table" + self.sfx)
+        self._table.argtypes = [vp]
+        self._bin = getattr(L, "orc_sigmoid_bin" + self.sfx)
+        self._bin.argtypes = [self.cv]
+        self._bin.restype = C.c_int
+        self._sop_array = getattr(L, "orc_sop_array" + self.sfx)
+        self._sop_array.argtypes = [C.c_int, vp, vp, C.c_int64]
+        self._gpu_dot = getattr(L, "orc_gpu_dot" + self.sfx)
+        self._gpu_dot.argtypes = [vp, vp, C.c_int64, C.c_int, C.c_int, C.c_int]
+        self._gpu_dot.restype = self.cv
         L.orc_max_threads.restype = C.c_int
 
     def table(self):
-        t = np.empty(2048, np.float32)
-        self.lib.orc_sigmoid_table(_ptr(t, C.c_float))
+        t = np.empty(2048, self.np_v)
+        self._table(_ptr(t, self.cv))
         return t
 
     def bin(self, v):
-        return self.lib.orc_sigmoid_bin(C.c_float(v))
+        return self._bin(self.cv(v))
 
     def sop(self, kind, arr):
-        a = np.ascontiguousarray(arr, np.float32)
+        a = np.ascontiguousarray(arr, self.np_v)
         out = np.empty_like(a)
-        self.lib.orc_sop_array(kind, _ptr(a, C.c_float), _ptr(out, C.c_float), a.size)
+        self._sop_array(kind, _ptr(a, self.cv), _ptr(out, self.cv), a.size)
         return out
 
     def gpu_dot(self, x, y, V, L, diff=0):
-        x = np.ascontiguousarray(x, np.float32)
-        y = np.ascontiguousarray(y, np.float32)
-        return self.lib.orc_gpu_dot(_ptr(x, C.c_float), _ptr(y, C.c_float), x.size, V, L, diff)
+        x = np.ascontiguousarray(x, self.np_v)
+        y = np.ascontiguousarray(y, self.np_v)
+        return self._gpu_dot(_ptr(x, self.cv), _ptr(y, self.cv), x.size, V, L, diff)
 
     def max_threads(self):
         return self.lib.orc_max_threads()
+
+    def _val(self, g):
+        """Edge values in this instance's precision (graphs carry float32 values)."""
+        v = g["val"]
+        return v if v is None or v.dtype == self.np_v else v.astype(self.np_v)
 
     def partition(self, pntrb, pntre, nthreads, m=None):
         bits = pntrb.dtype.itemsize * 8
@@ -92,18 +108,21 @@ class Oracle:
         m = len(pntrb) if m is None else m
         rb = np.empty(nthreads, np.int64)
         re = np.empty(nthreads, np.int64)
-        fn = getattr(self.lib, "orc_partition_rows_i%d" % bits)
+        fn = getattr(self.lib, "orc_partition_rows_i%d" % bits)   # value-type independent
         fn.argtypes = [ct, C.POINTER(ct), C.POINTER(ct), C.c_int, C.POINTER(C.c_int64), C.POINTER(C.c_int64)]
         fn.restype = C.c_int
         rc = fn(m, _ptr(pntrb, ct), _ptr(pntre, ct), nthreads, _ptr(rb, C.c_int64), _ptr(re, C.c_int64))
         return rc, rb, re
 
     @staticmethod
-    def _csr_args(ct, m, n, k, nnz, rows, cols, val, indx, pntrb, pntre, x, ldx, y, ldy, beta, z, ldz):
-        return [ct(m), ct(n), ct(k), C.c_float(1.0), ct(nnz), ct(rows), ct(cols),
-                _ptr(val, C.c_float), _ptr(indx, ct), _ptr(pntrb, ct), _ptr(pntre, ct),
-                _ptr(x, C.c_float), ct(ldx), _ptr(y, C.c_float), ct(ldy), C.c_float(beta),
-                _ptr(z, C.c_float), ct(ldz)]
+    def _csr_args(ct, m, n, k, nnz, rows, cols, val, indx, pntrb, pntre, x, ldx, y, ldy, beta, z, ldz, cv=C.c_float):
+        np_v = np.float32 if cv is C.c_float else np.float64
+        for a in (val, x, y, z):
+            assert a is None or a.dtype == np_v, "operand dtype does not match the library's VALUETYPE"
+        return [ct(m), ct(n), ct(k), cv(1.0), ct(nnz), ct(rows), ct(cols),
+                _ptr(val, cv), _ptr(indx, ct), _ptr(pntrb, ct), _ptr(pntre, ct),
+                _ptr(x, cv), ct(ldx), _ptr(y, cv), ct(ldy), cv(beta),
+                _ptr(z, cv), ct(ldz)]
 
     def generic(self, imsg, g, x, y, z, beta=0.0, sop_kind=0, m=None, k=None, ldx=None, ldy=None, ldz=None):
         """orc_fusedmm_generic; g is a graph dict (see tests/graphs.py). z is updated in place."""
@@ -114,11 +133,11 @@ class Oracle:
         ldx = (x.shape[1] if x is not None else k) if ldx is None else ldx
         ldy = y.shape[1] if ldy is None else ldy
         ldz = z.shape[1] if ldz is None else ldz
-        fn = getattr(self.lib, "orc_fusedmm_generic_i%d" % bits)
+        fn = getattr(self.lib, "orc_fusedmm_generic%s_i%d" % (self.sfx, bits))
         fn.restype = C.c_int
         args = [C.c_int32(imsg)] + self._csr_args(ct, m, g["cols"], k, g["nnz"], g["rows"], g["cols"],
-                                                  g["val"], g["indx"], g["pntrb"], g["pntre"],
-                                                  x, ldx, y, ldy, beta, z, ldz) + [C.c_int(sop_kind)]
+                                                  self._val(g), g["indx"], g["pntrb"], g["pntre"],
+                                                  x, ldx, y, ldy, beta, z, ldz, self.cv) + [C.c_int(sop_kind)]
         return fn(*args)
 
     def opt(self, tkern, g, x, y, z, beta=0.0, sop_kind=0, mode=0, V=4, L=32, S=1, m=None, k=None,
@@ -130,12 +149,12 @@ class Oracle:
         ldx = (x.shape[1] if x is not None else k) if ldx is None else ldx
         ldy = y.shape[1] if ldy is None else ldy
         ldz = z.shape[1] if ldz is None else ldz
-        fn = getattr(self.lib, "orc_fusedmm_opt_i%d" % bits)
+        fn = getattr(self.lib, "orc_fusedmm_opt%s_i%d" % (self.sfx, bits))
         fn.restype = C.c_int
         args = [C.c_char(tkern.encode())] + self._csr_args(ct, m, g["cols"], k, g["nnz"], g["rows"], g["cols"],
-                                                           g["val"], g["indx"], g["pntrb"], g["pntre"],
-                                                           x, ldx, y, ldy, beta, z, ldz)
-        args += [C.c_int(sop_kind), C.c_int(mode), C.c_int(V), C.c_int(L), C.c_int(S), _ptr(edge_s, C.c_float)]
+                                                           self._val(g), g["indx"], g["pntrb"], g["pntre"],
+                                                           x, ldx, y, ldy, beta, z, ldz, self.cv)
+        args += [C.c_int(sop_kind), C.c_int(mode), C.c_int(V), C.c_int(L), C.c_int(S), _ptr(edge_s, self.cv)]
         return fn(*args)
 
     def baseline(self, tkern, g, x, y, z, beta=0.0, sop_kind=0, nthreads=1, m=None):
@@ -143,46 +162,54 @@ class Oracle:
         _, ct = _itype(bits)
         m = g["rows"] if m is None else m
         k = y.shape[1]
-        fn = getattr(self.lib, "orc_fusedmm_baseline_i%d" % bits)
+        fn = getattr(self.lib, "orc_fusedmm_baseline%s_i%d" % (self.sfx, bits))
         fn.restype = C.c_int
         args = [C.c_char(tkern.encode())] + self._csr_args(ct, m, g["cols"], k, g["nnz"], g["rows"], g["cols"],
-                                                           g["val"], g["indx"], g["pntrb"], g["pntre"],
-                                                           x, x.shape[1] if x is not None else k, y, k, beta, z, k)
+                                                           self._val(g), g["indx"], g["pntrb"], g["pntre"],
+                                                           x, x.shape[1] if x is not None else k, y, k, beta, z, k,
+                                                           self.cv)
         args += [C.c_int(sop_kind), C.c_int(nthreads)]
         return fn(*args)
 
 
-def ref_available(kind="sigmoid", bits=32):
-    return os.path.exists(os.path.join(ORACLE_DIR, "_ref", "libref_%s_i%d.so" % (kind, bits)))
+def _ref_name(kind, bits, vbits):
+    return "libref_%s_%si%d.so" % (kind, "d_" if vbits == 64 else "", bits)
+
+
+def ref_available(kind="sigmoid", bits=32, vbits=32):
+    return os.path.exists(os.path.join(ORACLE_DIR, "_ref", _ref_name(kind, bits, vbits)))
 
 
 class Ref:
     """The real reference (harness + generic fusedMM_csr), one library per SOP body."""
 
-    def __init__(self, kind, bits=32):
+    def __init__(self, kind, bits=32, vbits=32):
         self.bits = bits
         self.np_i, self.ct = _itype(bits)
-        self.lib = C.CDLL(os.path.join(ORACLE_DIR, "_ref", "libref_%s_i%d.so" % (kind, bits)))
-        assert self.lib.ref_index_bytes() * 8 == bits
+        self.np_v, self.cv = _vtype(vbits)
+        self.lib = C.CDLL(os.path.join(ORACLE_DIR, "_ref", _ref_name(kind, bits, vbits)))
+        assert self.lib.ref_index_bytes() * 8 == bits and self.lib.ref_value_bytes() * 8 == vbits
 
     def table(self):
-        t = np.empty(2048, np.float32)
-        self.lib.ref_sm_table(_ptr(t, C.c_float))
+        t = np.empty(2048, self.np_v)
+        self.lib.ref_sm_table(_ptr(t, self.cv))
         return t
 
     def sop(self, arr):
-        a = np.ascontiguousarray(arr, np.float32)
+        a = np.ascontiguousarray(arr, self.np_v)
         out = np.empty_like(a)
-        self.lib.ref_sop_array.argtypes = [_f32p, _f32p, C.c_int64]
-        self.lib.ref_sop_array(_ptr(a, C.c_float), _ptr(out, C.c_float), a.size)
+        vp = C.POINTER(self.cv)
+        self.lib.ref_sop_array.argtypes = [vp, vp, C.c_int64]
+        self.lib.ref_sop_array(_ptr(a, self.cv), _ptr(out, self.cv), a.size)
         return out
 
     def _call(self, fn, head, g, x, y, z, beta, m):
         ct = self.ct
         m = g["rows"] if m is None else m
         k = y.shape[1]
-        args = head + Oracle._csr_args(ct, m, g["cols"], k, g["nnz"], g["rows"], g["cols"], g["val"], g["indx"],
-                                       g["pntrb"], g["pntre"], x, k, y, k, beta, z, k)
+        val = g["val"] if g["val"] is None or g["val"].dtype == self.np_v else g["val"].astype(self.np_v)
+        args = head + Oracle._csr_args(ct, m, g["cols"], k, g["nnz"], g["rows"], g["cols"], val, g["indx"],
+                                       g["pntrb"], g["pntre"], x, k, y, k, beta, z, k, self.cv)
         return fn(*args)
 
     def trusted(self, tkern, g, x, y, z, beta=0.0, m=None):
@@ -202,6 +229,6 @@ class Ref:
         self.lib.ref_load_mtx(path.encode(), C.byref(r), C.byref(c), C.byref(n))
         rowptr = np.empty(r.value + 1, self.np_i)
         colids = np.empty(n.value, self.np_i)
-        values = np.empty(n.value, np.float32)
-        self.lib.ref_get_csr(_ptr(rowptr, self.ct), _ptr(colids, self.ct), _ptr(values, C.c_float))
+        values = np.empty(n.value, self.np_v)
+        self.lib.ref_get_csr(_ptr(rowptr, self.ct), _ptr(colids, self.ct), _ptr(values, self.cv))
         return r.value, c.value, rowptr, colids, values

@@ -17,20 +17,24 @@ def declared_entry_points():
     for h in ("fusedMM.h", "fusedmm_amd.h"):
         text = open(os.path.join(ROOT, "include", h)).read()
         text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
-        names |= set(re.findall(r"\b((?:fusedMM_|sgfusedMM_)\w+)\s*\(", text))
+        names |= set(re.findall(r"\b((?:fusedMM_|sgfusedMM_|dgfusedMM_)\w+)\s*\(", text))
     names.discard("fusedMM_amd_sop_fn")
     return sorted(names)
 
 
+@pytest.mark.parametrize("vbits", [32, 64])
 @pytest.mark.parametrize("bits", [32, 64])
-def test_library_exports_declared_symbols(bits):
-    lib = fa.load(bits)
+def test_library_exports_declared_symbols(bits, vbits):
+    lib = fa.load(bits, vbits)
     names = declared_entry_points()
-    assert "fusedMM_csr" in names and "fusedMM_csr_stream" in names and len(names) >= 12
+    assert "fusedMM_csr" in names and "fusedMM_csr_stream" in names and len(names) >= 14
+    # the second-level entry is named after the precision, as in the reference (kernels.h:17-37)
+    own, other = ("sgfusedMM_csr", "dgfusedMM_csr") if vbits == 32 else ("dgfusedMM_csr", "sgfusedMM_csr")
     for n in names:
-        assert hasattr(lib, n), n
-    assert set(names) == set(fa.EXPORTS)
-    assert lib.fusedMM_amd_index_bytes() * 8 == bits
+        if n != other:
+            assert hasattr(lib, n), n
+    assert set(names) == set(fa.EXPORTS) | {own, other}
+    assert lib.fusedMM_amd_index_bytes() * 8 == bits and lib.fusedMM_amd_value_bytes() * 8 == vbits
 
 
 def test_header_constants_match_python_mirror():

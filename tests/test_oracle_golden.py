@@ -72,3 +72,49 @@ def test_tuple_sweep_bit_equal(oracle):
         if (int(imsg) & 0xF00) == 0x000 and (int(imsg) & 0xF000) != 0:
             continue   # SOP_NOOP feeding a VSC reads an uninitialised scalar in the reference
         assert bits_equal(Z, want), hex(int(imsg))
+
+
+# ---- double precision (the reference's -DDREAL build) ------------------------------------
+
+def bits_equal64(a, b):
+    return np.array_equal(np.asarray(a, np.float64).view(np.uint64), np.asarray(b, np.float64).view(np.uint64))
+
+
+@pytest.fixture(scope="module")
+def oracle_d():
+    from oracle_api import Oracle
+    return Oracle(vbits=64)
+
+
+def test_double_table_and_sop_bodies_bit_equal(oracle_d):
+    d = np.load(os.path.join(GOLD, "sop.npz"))
+    assert bits_equal64(oracle_d.table(), d["table_d"])
+    v = d["probe_d"]
+    for kind in ("sigmoid", "tdist", "fr", "ll", "fa"):
+        arg = v if kind == "sigmoid" else np.abs(v) + 1e-3
+        assert bits_equal64(oracle_d.sop(SOP_NAMES[kind], arg), d["sop_%s_d" % kind]), kind
+
+
+@pytest.mark.parametrize("bits", [32, 64])
+@pytest.mark.parametrize("t", ["s", "t", "f", "m", "g"])
+def test_double_ops_against_reference(oracle_d, bits, t):
+    d = np.load(os.path.join(GOLD, "ops_d_i%d.npz" % bits))
+    g = graph_from(d, "ragged", bits)
+    k = 24
+    X, Y = d["ragged_X%d" % k], d["ragged_Y%d" % k]
+    sk = SOP_NAMES[KIND_OF[t]] if KIND_OF[t] else 0
+    want_f = d["ragged_%s_k%d_fusedmm" % (t, k)]
+    want_t = d["ragged_%s_k%d_trusted" % (t, k)]
+    Z = np.zeros_like(want_f)
+    assert oracle_d.generic(MSG[t], g, X, Y, Z, sop_kind=sk) == 0
+    assert bits_equal64(Z, want_f)
+    ot = "t" if t == "f" else t
+    Z = np.zeros_like(want_f)
+    assert oracle_d.opt(ot, g, X, Y, Z, beta=0.0, sop_kind=sk, mode=0) == 0
+    assert bits_equal64(Z, want_f)
+    scale = np.abs(want_t).max() + 1.0
+    for mode in (1, 2):
+        Z = np.zeros_like(want_f)
+        oracle_d.opt(ot, g, X, Y, Z, beta=0.0, sop_kind=sk, mode=mode, V=4, L=8, S=8)
+        tol = 2e-3 if t == "s" else 1e-13          # sigmoid: a table-bin flip; otherwise rounding
+        assert np.abs(Z - want_t).max() <= tol * scale, (mode, np.abs(Z - want_t).max())

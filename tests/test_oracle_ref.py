@@ -50,3 +50,24 @@ def test_generic_path_bits(oracle, bits, t, k):
         r.test(t, g, X, Y, A, m=g["rows"] // 2)
         oracle.generic(MSG[t], g, X, Y, B, sop_kind=sk, m=g["rows"] // 2)
         assert bits_equal(A, B)
+
+
+@pytest.mark.skipif(not ref_available("sigmoid", 32, 64), reason="double-precision reference not built")
+@pytest.mark.parametrize("bits", [32, 64])
+@pytest.mark.parametrize("t", ["s", "t", "f", "m", "g"])
+def test_double_generic_path_bits(bits, t):
+    from oracle_api import Oracle
+    od = Oracle(vbits=64)
+    kind = KIND_OF[t]
+    r = Ref(kind, bits, 64)
+    sk = SOP_NAMES.get(kind, 0)
+    g = graphs.with_values(graphs.tiny_er(300, 2500, 4, bits))
+    for k in (8, 33):
+        X = graphs.features(g["rows"], k, 1, -1, 1, 1).astype(np.float64)
+        Y = graphs.features(g["cols"], k, 1, -1, 1, 2).astype(np.float64)
+        Z0 = graphs.features(g["rows"], k, 1, -1, 1, 3).astype(np.float64)
+        A, B = Z0.copy(), Z0.copy()
+        r.test(t, g, X, Y, A)
+        assert od.generic(MSG[t], g, X, Y, B, sop_kind=sk) == 0
+        assert np.array_equal(A.view(np.uint64), B.view(np.uint64))
+    assert np.array_equal(od.table().view(np.uint64), Ref("sigmoid", bits, 64).table().view(np.uint64))
