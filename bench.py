@@ -104,6 +104,8 @@ def main():
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--workload", default="c2", choices=sorted(WORKLOADS))
+    ap.add_argument("--dtype", default="f32", choices=["f32", "f64"],
+                    help="f64 runs the double-precision library (the reference's -DDREAL build)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-check", action="store_true", help="skip the spot check against the oracle")
     ap.add_argument("--copy-probe", action="store_true",
@@ -120,13 +122,20 @@ def main():
 
     desc, tkern, k, kind = WORKLOADS[args.workload]
     bits = 32
-    lib = fa.load(bits)
+    vbits = 32 if args.dtype == "f32" else 64
+    np_v = np.float32 if vbits == 32 else np.float64
+    lib = fa.load(bits, vbits)
     kind_id = {None: 0, "sigmoid": 1, "tdist": 2, "fr": 3}[kind]
     lib.fusedMM_amd_set_sop_kind(kind_id)
     imsg = {"s": fa.MSG_SIGMOID, "t": fa.MSG_TDIST, "f": fa.MSG_FR, "m": fa.MSG_SPMM, "g": fa.MSG_GCN}[tkern]
 
     t_gen = time.time()
     g, X, Y = make_workload(args.workload)
+    if vbits == 64:
+        same = Y is X
+        X = None if X is None else X.astype(np_v)
+        Y = X if same else Y.astype(np_v)
+        g["val"] = g["val"].astype(np_v)
     t_gen = time.time() - t_gen
     m, n, nnz = g["rows"], g["cols"], g["nnz"]
 
@@ -135,12 +144,12 @@ def main():
     d_val, d_indx, d_pb, d_pe = up(g["val"]), up(g["indx"]), up(g["pntrb"]), up(g["pntre"])
     d_X = up(X)
     d_Y = d_X if Y is X else up(Y)
-    d_Z = torch.zeros((m, k), dtype=torch.float32, device=dev)
+    d_Z = torch.zeros((m, k), dtype=torch.float32 if vbits == 32 else torch.float64, device=dev)
     stream = torch.cuda.current_stream().cuda_stream
 
     def step():
         rc = fa.fusedMM_csr(imsg, m, n, k, 1.0, nnz, m, n, d_val, d_indx, d_pb, d_pe, d_X, k, d_Y, k, 0.0, d_Z, k,
-                            index_bits=bits, stream=stream)
+                            index_bits=bits, stream=stream, value_bits=vbits)
         if rc != 0:
             raise SystemExit("fusedMM_csr returned %d" % rc)
 
@@ -167,7 +176,7 @@ def main():
     ms_per_step = wall / args.steps * 1e3
 
     flops = synth.algorithmic_flops(tkern, k, nnz)
-    b_alg = synth.algorithmic_bytes(tkern, m, k, nnz, 4)
+    b_alg = synth.algorithmic_bytes(tkern, m, k, nnz, 4, value_bytes=vbits // 8)
     value = flops / (ms_per_step * 1e-3) / 1e9
 
     kern_ms = {"rows_kernel": r_ms.value / max(1, ncalls), "segments_kernel": s_ms.value / max(1, ncalls),
@@ -182,7 +191,7 @@ def main():
     dom_ms = sum(kern_ms.values()) if split else kern_ms["rows_kernel"]
     achieved = b_alg / (dom_ms * 1e-3) / 1e9 if dom_ms > 0 else 0.0
     roofline = {"bound": "hbm", "achieved": achieved, "peak": PEAK_HBM_GBPS, "unit": "GB/s",
-                "frac": achieved / PEAK_HBM_GBPS, "traffic": MEASURED_TRAFFIC_BYTES.get(args.workload),
+                "frac": achieved / PEAK_HBM_GBPS, "traffic": MEASURED_TRAFFIC_BYTES.get(args.workload) if vbits == 32 else None,
                 "kernel": "rows_kernel+segments_kernel+merge_kernel" if split else "rows_kernel",
                 "kernel_ms": dom_ms, "algorithmic_bytes": b_alg}
 
@@ -194,8 +203,8 @@ def main():
         sys.path.insert(0, os.path.join(ROOT, "tests"))
         from oracle_api import Oracle
         from gpu_api import oracle_mirror, default_split
-        orc = Oracle()
-        heavy_deg, seg_len = default_split(k)
+        orc = Oracle(vbits=vbits)
+        heavy_deg, seg_len = default_split(k, vbits)
         deg = np.diff(g["rowptr"])
         windows = [(m // 2, min(m, m // 2 + 1024))]
         hub = int(np.argmax(deg))
@@ -207,16 +216,16 @@ def main():
             sub = dict(g)
             sub.update(rows=hi - lo, pntrb=g["pntrb"][lo:hi], pntre=g["pntre"][lo:hi])
             Xs = None if X is None else X[lo:hi]
-            want = oracle_mirror(orc, tkern, sub, Xs, Y, np.zeros((hi - lo, k), np.float32), 0.0, kind_id, k,
+            want = oracle_mirror(orc, tkern, sub, Xs, Y, np.zeros((hi - lo, k), np_v), 0.0, kind_id, k,
                                  heavy_deg, seg_len)
             got = z_all[lo:hi] if z_all is not None else d_Z[lo:hi].cpu().numpy()
-            checked = checked and bool(np.array_equal(got.view(np.uint32), want.view(np.uint32)))
+            checked = checked and bool(np.array_equal(got.view(np.uint8), want.view(np.uint8)))
 
     out = {
         "metric": "GFLOP/s + HBM GB/s (% of peak), sigmoid K=128, 1 MI355X vs CPU OpenMP",
         "value": value, "unit": "GFLOP/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": ms_per_step, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
-        "dtype": "f32", "data": "synthetic",
+        "dtype": args.dtype, "data": "synthetic",
         "config": {"workload": "%s: %s" % (args.workload, desc), "op": tkern, "K": k, "rows": m, "nnz": nnz,
                    "index_bits": bits, "beta": 0.0, "graph_gen_s": round(t_gen, 2)},
         "edges_per_s": nnz / (ms_per_step * 1e-3),
@@ -227,7 +236,7 @@ def main():
         "spot_check_vs_oracle": checked,
         "roofline": roofline,
     }
-    if not args.no_cpu:
+    if not args.no_cpu and vbits == 32:
         out["cpu_baseline"] = cpu_baseline(args.workload, g, X, Y, tkern, kind_id, k)
     print(json.dumps(out))
 

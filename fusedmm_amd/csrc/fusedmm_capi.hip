@@ -321,8 +321,11 @@ struct Args {
    val_t beta;
 };
 
-// Everything here is device memory.  Enqueues on `stream`, does not wait.
-int run_on_device(const Args &a, const Plan &pl, int sop_kind, hipStream_t stream)
+int run_on_device(const Args &a, const Plan &pl, int sop_kind, hipStream_t stream);
+
+// One call of the kernels, k <= kMaxK.  Everything here is device memory.
+// Enqueues on `stream`, does not wait.
+int run_slab(const Args &a, const Plan &pl, int sop_kind, hipStream_t stream)
 {
    if (a.m <= 0) return FUSEDMM_SUCCESS_RETURN;
    if (a.k < 1) return FUSEDMM_SUCCESS_RETURN;
@@ -522,24 +525,140 @@ int run_staged(const Args &h, const Plan &pl, int sop_kind)
 // scalars as edge values.  Synchronous; device operands `a`, host copies of
 // the row pointers in h_pb / h_pe.
 template <int V, int L, int R, bool EXACT, int U>
-int launch_edge_scalar(const Params<idx_t> &p, val_t *s_out, int num_cu)
+int launch_edge_scalar(const Params<idx_t> &p, val_t *s_out, int accumulate, int num_cu, hipStream_t stream)
 {
    int64_t blocks = (p.m + kWavesPerBlock - 1) / kWavesPerBlock;
    if (blocks > (int64_t)num_cu * 8) blocks = (int64_t)num_cu * 8;
-   hipLaunchKernelGGL((edge_scalar_kernel<V, L, R, EXACT, U, idx_t>), dim3((unsigned int)blocks), dim3(kBlockThreads), 0, 0,
-                      p, s_out);
+   hipLaunchKernelGGL((edge_scalar_kernel<V, L, R, EXACT, U, idx_t>), dim3((unsigned int)blocks), dim3(kBlockThreads), 0,
+                      stream, p, s_out, accumulate);
    return hip_status(hipGetLastError(), "edge scalar launch");
+}
+
+// d_s[j] = ROP(X[i], VOP(X[i], Y[c])) for every edge slot of the processed rows,
+// column slab by column slab when k exceeds what one kernel instance holds.
+int edge_scalars(const Args &a, val_t *d_s, DeviceState *d, hipStream_t stream)
+{
+   constexpr int64_t ld_mult = 16 / (int64_t)kValBytes;
+   for (int64_t off = 0; off < a.k; off += kMaxK)
+   {
+      const int64_t ks = a.k - off < kMaxK ? a.k - off : kMaxK;
+      const val_t *xs = a.x ? a.x + off : nullptr, *ys = a.y + off;
+      const bool vec_ok = (ks % 4 == 0) && (a.ldy % ld_mult == 0) && aligned16(ys) && (!xs || ((a.ldx % ld_mult == 0) && aligned16(xs)));
+      Shape sh;
+      int st = pick_shape((int)ks, vec_ok, &sh);
+      if (st) return st;
+      Params<idx_t> p;
+      memset(&p, 0, sizeof(p));
+      p.pntrb = a.pntrb; p.pntre = a.pntre; p.indx = a.indx; p.val = a.val;
+      p.x = xs ? xs : ys;   // tuples that never read X still index it; any valid row will do
+      p.y = ys; p.m = a.m; p.ldx = xs ? a.ldx : 0; p.ldy = a.ldy; p.k = (int)ks; p.imessage = a.imessage;
+      st = FUSEDMM_FAIL_RETURN;
+#define FMM_CASE(V_, L_, R_, X_, U_) \
+   if (sh.V == V_ && sh.L == L_ && sh.R == R_ && sh.exact == X_) \
+      st = launch_edge_scalar<V_, L_, R_, (X_ != 0), U_>(p, d_s, off > 0 ? 1 : 0, d->num_cu, stream);
+      FMM_SHAPES(FMM_CASE)
+#undef FMM_CASE
+      if (st) return st;
+   }
+   return FUSEDMM_SUCCESS_RETURN;
+}
+
+int64_t max_slot(const idx_t *h_pe, int64_t m)
+{
+   int64_t slots = 0;
+   for (int64_t i = 0; i < m; i++)
+      if ((int64_t)h_pe[i] > slots) slots = (int64_t)h_pe[i];
+   return slots;
+}
+
+bool column_separable(const Plan &pl, int32_t imsg)
+{
+   return pl.op == OP_GCN || pl.op == OP_SPMM || (pl.op == OP_GENERIC && GET_ROP_FLAG(imsg) == ROP_NOOP);
+}
+
+// Rest of the pipeline (VOP, MOP, AOP) with per-edge scalars already in d_s.
+int accumulate_with_scalars(const Args &a, val_t *d_s, hipStream_t stream)
+{
+   Args a2 = a;
+   a2.val = d_s;
+   a2.imessage = GET_VOP_FLAG(a.imessage) | ROP_NOOP | SOP_COPY | GET_VSC_FLAG(a.imessage) | GET_AOP_FLAG(a.imessage);
+   Plan p2;
+   int st = make_plan(a2.imessage, 0, &p2);   // general rule: accumulate (Z is cleared first when it must be overwritten)
+   if (st) return st;
+   return run_on_device(a2, p2, FUSEDMM_SOP_KIND_IDENTITY, stream);
+}
+
+// k > kMaxK with a reduction over the whole row (dot / distance tuples): the
+// per-edge scalar is assembled from column slabs, the device SOP applied to it,
+// then the accumulate stage runs slab by slab.  Synchronous (needs the largest
+// edge slot, read back from the row pointers).
+int run_wide_reduction(const Args &a, const Plan &pl, int sop_kind)
+{
+   DeviceState *d = nullptr;
+   int st = device_state(&d);
+   if (st) return st;
+   std::vector<idx_t> he((size_t)a.m);
+   FMM_HIP(hipMemcpy(he.data(), a.pntre, (size_t)a.m * sizeof(idx_t), hipMemcpyDeviceToHost));
+   const int64_t slots = max_slot(he.data(), a.m);
+   if (pl.opt_rule && a.beta == 0.0f)
+      FMM_HIP(hipMemset2DAsync(a.z, (size_t)a.ldz * kValBytes, 0, (size_t)a.k * kValBytes, (size_t)a.m, 0));
+   if (slots <= 0) return FUSEDMM_SUCCESS_RETURN;
+   st = grow(d->stage[7], (size_t)slots * kValBytes);
+   if (st) return st;
+   val_t *d_s = (val_t *)d->stage[7].ptr;
+   st = edge_scalars(a, d_s, d, 0);
+   if (st) return st;
+   if (pl.needs_sop)
+   {
+      hipLaunchKernelGGL(apply_sop_kernel, dim3((unsigned int)(d->num_cu * 4)), dim3(kBlockThreads), 0, 0, d_s, slots,
+                         sop_kind, (const val_t *)d->sigmoid_table);
+      st = hip_status(hipGetLastError(), "apply sop launch");
+      if (st) return st;
+   }
+   return accumulate_with_scalars(a, d_s, 0);
+}
+
+// Everything here is device memory.  Enqueues on `stream`, does not wait
+// (except for wide rows with a whole-row reduction, see run_wide_reduction).
+int run_on_device(const Args &a, const Plan &pl, int sop_kind, hipStream_t stream)
+{
+   if (a.m <= 0 || a.k < 1) return FUSEDMM_SUCCESS_RETURN;
+   if (a.k <= kMaxK) return run_slab(a, pl, sop_kind, stream);
+   if (a.ldy < a.k || a.ldz < a.k || (pl.reads_x && a.ldx < a.k))
+   {
+      FMM_LOG("leading dimension smaller than k");
+      return FUSEDMM_FAIL_RETURN;
+   }
+   if (column_separable(pl, a.imessage))
+   {
+      // no stage looks across columns: every slab of kMaxK columns is a call of its own
+      for (int64_t off = 0; off < a.k; off += kMaxK)
+      {
+         Args s = a;
+         s.k = a.k - off < kMaxK ? a.k - off : kMaxK;
+         s.x = a.x ? a.x + off : nullptr;
+         s.y = a.y + off;
+         s.z = a.z + off;
+         int st = run_slab(s, pl, sop_kind, stream);
+         if (st) return st;
+      }
+      return FUSEDMM_SUCCESS_RETURN;
+   }
+   if (stream != 0)
+   {
+      FMM_LOG("k=%lld with a whole-row reduction needs the synchronous entry point", (long long)a.k);
+      return FUSEDMM_FAIL_RETURN;
+   }
+   return run_wide_reduction(a, pl, sop_kind);
 }
 
 int run_host_sop(const Args &a, const idx_t *h_pb, const idx_t *h_pe, int64_t slots, const Plan &pl,
                  fusedMM_amd_sop_fn fn)
 {
    if (a.m <= 0 || a.k < 1) return FUSEDMM_SUCCESS_RETURN;
-   if (a.k > kMaxK) { FMM_LOG("feature dimension k=%lld is beyond the supported maximum %d", (long long)a.k, kMaxK); return FUSEDMM_FAIL_RETURN; }
    DeviceState *d = nullptr;
    int st = device_state(&d);
    if (st) return st;
-   const int vsc = GET_VSC_FLAG(a.imessage);
    const bool overwrite = pl.opt_rule && a.beta == 0.0f;
    if (overwrite)
       FMM_HIP(hipMemset2DAsync(a.z, (size_t)a.ldz * kValBytes, 0, (size_t)a.k * kValBytes, (size_t)a.m, 0));
@@ -549,21 +668,7 @@ int run_host_sop(const Args &a, const idx_t *h_pb, const idx_t *h_pe, int64_t sl
    val_t *d_s = (val_t *)d->stage[7].ptr;
 
    // pass 1
-   constexpr int64_t ld_mult = 16 / (int64_t)kValBytes;
-   const bool vec_ok = (a.k % 4 == 0) && (a.ldy % ld_mult == 0) && aligned16(a.y) && (a.ldx % ld_mult == 0) && aligned16(a.x);
-   Shape sh;
-   st = pick_shape((int)a.k, vec_ok, &sh);
-   if (st) return st;
-   Params<idx_t> p;
-   memset(&p, 0, sizeof(p));
-   p.pntrb = a.pntrb; p.pntre = a.pntre; p.indx = a.indx; p.val = a.val;
-   p.x = a.x ? a.x : a.y;   // tuples that never read X still index it; any valid row will do
-   p.y = a.y; p.m = a.m; p.ldx = a.x ? a.ldx : 0; p.ldy = a.ldy; p.k = (int)a.k; p.imessage = a.imessage;
-   st = FUSEDMM_FAIL_RETURN;
-#define FMM_CASE(V_, L_, R_, X_, U_) \
-   if (sh.V == V_ && sh.L == L_ && sh.R == R_ && sh.exact == X_) st = launch_edge_scalar<V_, L_, R_, (X_ != 0), U_>(p, d_s, d->num_cu);
-   FMM_SHAPES(FMM_CASE)
-#undef FMM_CASE
+   st = edge_scalars(a, d_s, d, 0);
    if (st) return st;
    std::vector<val_t> hs((size_t)slots);
    FMM_HIP(hipMemcpyAsync(hs.data(), d_s, (size_t)slots * kValBytes, hipMemcpyDeviceToHost, 0));
@@ -590,13 +695,7 @@ int run_host_sop(const Args &a, const idx_t *h_pb, const idx_t *h_pe, int64_t sl
    FMM_HIP(hipMemcpyAsync(d_s, hs.data(), (size_t)slots * kValBytes, hipMemcpyHostToDevice, 0));
 
    // pass 2: same VOP / MOP / AOP, the scalar comes in as the edge value
-   Args a2 = a;
-   a2.val = d_s;
-   a2.imessage = GET_VOP_FLAG(a.imessage) | ROP_NOOP | SOP_COPY | vsc | GET_AOP_FLAG(a.imessage);
-   Plan p2;
-   st = make_plan(a2.imessage, 0, &p2);   // general rule: accumulate (Z was cleared above when it must be overwritten)
-   if (st) return st;
-   st = run_on_device(a2, p2, FUSEDMM_SOP_KIND_IDENTITY, 0);
+   st = accumulate_with_scalars(a, d_s, 0);
    if (st) return st;
    return hip_status(hipStreamSynchronize(0), "hipStreamSynchronize");
 }

@@ -958,7 +958,7 @@ __global__ __launch_bounds__(kBlockThreads) void merge_kernel(const Params<IdxT>
 // One wave per row (static stride; this path exists for compatibility, the
 // host evaluates the caller's SOP_UDEF_FUNC on s[] before the accumulate pass).
 template <int V, int L, int R, bool EXACT, int U, typename IdxT>
-__global__ __launch_bounds__(kBlockThreads) void edge_scalar_kernel(const Params<IdxT> p, real_t *s_out)
+__global__ __launch_bounds__(kBlockThreads) void edge_scalar_kernel(const Params<IdxT> p, real_t *s_out, int accumulate)
 {
    constexpr int S = 64 / L;
    const int lane = threadIdx.x & 63;
@@ -983,11 +983,20 @@ __global__ __launch_bounds__(kBlockThreads) void edge_scalar_kernel(const Params
                Slice<R> ys, t;
                load_slice<V, L, R, EXACT>(ys, p.y + (int64_t)p.indx[j] * p.ldy, sl, p.k);
                const real_t scal = vop_rop<L, R>(t, xs, ys, p.val ? p.val[j] : (real_t)0, vop, rop);
-               if (sl == 0) s_out[j] = scal;
+               // every ROP is a sum over elements, so column slabs of a wide row add up
+               if (sl == 0) s_out[j] = accumulate ? s_out[j] + scal : scal;
             }
          }
       }
    }
+}
+
+// d[j] = SOP(s[j]) in place, for the wide-row path where the ROP result is
+// assembled from column slabs before the scalar op can be applied.
+__global__ __launch_bounds__(kBlockThreads) void apply_sop_kernel(real_t *s, int64_t n, int sop_kind, const real_t *tab)
+{
+   for (int64_t i = (int64_t)blockIdx.x * kBlockThreads + threadIdx.x; i < n; i += (int64_t)gridDim.x * kBlockThreads)
+      s[i] = sop_eval(sop_kind, s[i], tab);
 }
 
 // Clears the queue and claim counters before each call.  A kernel rather than a

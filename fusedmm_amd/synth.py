@@ -158,11 +158,11 @@ def write_mtx_symmetric(path, g):
         np.savetxt(f, np.stack([r, c], 1), fmt="%d")
 
 
-def algorithmic_bytes(kind, m, k, nnz, index_bytes=4, beta_nonzero=False):
+def algorithmic_bytes(kind, m, k, nnz, index_bytes=4, beta_nonzero=False, value_bytes=4):
     """Bytes one call must move if nothing is reused: every edge gathers a full
     Y row plus its column id (and value for spmm); every row reads X once (ops
     that use X), both row pointers, and writes Z once."""
-    F = 4
+    F = value_bytes
     vb = F if kind == "m" else 0
     xb = F * k if kind in ("s", "t", "f") else 0
     zb = F * k * (2 if beta_nonzero else 1)

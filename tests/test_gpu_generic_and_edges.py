@@ -137,12 +137,25 @@ def test_empty_inputs():
     assert rc == 0 and np.array_equal(Z, Z0)          # m == 0: nothing happens
 
 
-def test_k_beyond_supported_maximum_is_an_error():
-    g = graphs.tiny_er(20, 30, 2)
-    k = 2052
-    Y = np.zeros((20, k), np.float32)
-    rc, _ = gpu_api.run(MSG["g"], g, None, Y, np.zeros((20, k), np.float32))
-    assert rc == fa.FAIL
+@pytest.mark.parametrize("k", [2052, 4100, 2049])
+@pytest.mark.parametrize("tkern,kind", [("g", None), ("m", None), ("s", "sigmoid"), ("t", "tdist")])
+def test_rows_wider_than_one_kernel_instance(oracle, tkern, kind, k):
+    """k > 2048: processed in column slabs of 2048; tuples that reduce over the
+    whole row assemble the per-edge scalar from the slabs first."""
+    g = graphs.ragged(32, rows=40, cols=60, hub_deg=300)
+    amp = 0.05 if tkern in ("s", "t") else 0.5          # keep dots inside the sigmoid table's range
+    X = graphs.features(g["rows"], k, 4, -amp, amp, 1)
+    Y = graphs.features(g["cols"], k, 4, -amp, amp, 2)
+    Z0 = graphs.features(g["rows"], k, 4, -1, 1, 3)
+    sk = SOP_NAMES[kind] if kind else 0
+    gpu_api.set_kind(sk, 32)
+    for beta, where in ((0.0, "device"), (1.0, "host")):
+        rc, Z = gpu_api.run(MSG[tkern], g, X, Y, Z0, beta=beta, bits=32, where=where)
+        assert rc == 0
+        want = Z0.copy()
+        oracle.opt(tkern, g, X, Y, want, beta=beta, sop_kind=sk, mode=1)
+        extra = checks.sigmoid_flip_slack(oracle.table(), g, X, Y)[0] if tkern == "s" else None
+        checks.assert_close(Z, want, 1e-4, 1e-5, extra, "%s k=%d" % (tkern, k))
 
 
 @pytest.mark.parametrize("bits", [32, 64])
