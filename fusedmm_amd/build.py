@@ -48,8 +48,8 @@ def build_one(index_bits, value_bits=32, verbose=False):
     return out
 
 
-def timer_path(index_bits):
-    return os.path.join(HERE, "bin", "xfusedMMtime_i%d" % index_bits)
+def timer_path(index_bits, value_bits=32):
+    return os.path.join(HERE, "bin", "xfusedMMtime_%si%d" % ("d_" if value_bits == 64 else "", index_bits))
 
 
 def dropin_path(index_bits):
@@ -72,10 +72,14 @@ def _run(cmd, verbose):
 def build_timer(index_bits, verbose=False):
     """The tester/timer executable (csrc/fusedMMtime.cpp) and the loader's C doorway."""
     os.makedirs(os.path.join(HERE, "bin"), exist_ok=True)
+    for vbits in (32, 64):
+        exe_v = timer_path(index_bits, vbits)
+        _run([HIPCC, "-O2", "-std=c++17", "-fopenmp", "-DINDEXTYPE=int%d_t" % index_bits] +
+             (["-DDREAL"] if vbits == 64 else []) +
+             [os.path.join(CSRC, "fusedMMtime.cpp"), "-o", exe_v, "-L" + HERE,
+              "-l" + lib_name(index_bits, vbits)[3:-3],
+              "-Wl,-rpath,$ORIGIN/..", "-L/opt/rocm/lib", "-lrocprofiler-sdk-roctx", "-Wl,-rpath,/opt/rocm/lib"], verbose)
     exe = timer_path(index_bits)
-    _run([HIPCC, "-O2", "-std=c++17", "-fopenmp", "-DINDEXTYPE=int%d_t" % index_bits,
-          os.path.join(CSRC, "fusedMMtime.cpp"), "-o", exe, "-L" + HERE, "-lfusedmm_amd_i%d" % index_bits,
-          "-Wl,-rpath,$ORIGIN/..", "-L/opt/rocm/lib", "-lrocprofiler-sdk-roctx", "-Wl,-rpath,/opt/rocm/lib"], verbose)
     _run(["g++", "-O2", "-std=c++17", "-fPIC", "-shared", "-DINDEXTYPE=int%d_t" % index_bits,
           os.path.join(CSRC, "harness_capi.cpp"), "-o", harness_lib_path(index_bits)], verbose)
     # a reference-style caller in plain C (gcc, host pointers, its own SOP_UDEF_FUNC)

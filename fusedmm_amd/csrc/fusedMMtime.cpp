@@ -38,12 +38,17 @@
 #ifndef INDEXTYPE
 #define INDEXTYPE int64_t
 #endif
+#ifdef DREAL       /* double precision, as in the reference's build (-DDREAL) */
+#define VALUETYPE double
+#else
 #define VALUETYPE float
+#endif
 #include "../../include/fusedMM.h"
 #include "../../include/fusedmm_amd.h"
 #include "mtx_csr.hpp"
 
 typedef INDEXTYPE IT;
+typedef VALUETYPE VT;
 
 static bool g_prof = false;
 struct Range {
@@ -61,62 +66,63 @@ struct Range {
    } while (0)
 
 // ---- trusted (scalar) kernels ---------------------------------------------------------
-static float g_table[2048];
+static VT g_table[2048];
 static void init_table()
 {
    for (int i = 0; i < 2048; i++)
    {
-      float x = (float)(2.0 * 5.0 * i / 2048 - 5.0);
-      g_table[i] = (float)(1.0 / (double)(1 + expf(-x)));
+      VT x = (VT)(2.0 * 5.0 * i / 2048 - 5.0);
+      VT e = std::exp(-x);               // overload of VALUETYPE, as in the reference's C++ tester
+      g_table[i] = (VT)(1.0 / (double)(1 + e));
    }
 }
-static inline float table_sigmoid(float v)
+static inline VT table_sigmoid(VT v)
 {
-   if (v > 5.0f) return 1.0f;
-   if (v < -5.0f) return 0.0f;
+   if (v > 5.0) return 1.0;
+   if (v < -5.0) return 0.0;
    int i = (int)(((double)v + 5.0) * 2048 / 10.0);
    return g_table[i > 2047 ? 2047 : i];
 }
 
-static void trusted(char tkern, IT m, IT k, const float *val, const IT *indx, const IT *pntrb, const IT *pntre,
-                    const float *a, const float *b, float *c)
+static void trusted(char tkern, IT m, IT k, const VT *val, const IT *indx, const IT *pntrb, const IT *pntre,
+                    const VT *a, const VT *b, VT *c)
 {
 #pragma omp parallel for schedule(dynamic, 64)
    for (IT i = 0; i < m; i++)
    {
-      std::vector<float> T((size_t)k);
-      float *ci = c + (int64_t)i * k;
-      const float *ai = a + (int64_t)i * k;
+      std::vector<VT> T((size_t)k);
+      VT *ci = c + (int64_t)i * k;
+      const VT *ai = a + (int64_t)i * k;
       for (IT j = pntrb[i]; j < pntre[i]; j++)
       {
-         const float *bj = b + (int64_t)indx[j] * k;
+         const VT *bj = b + (int64_t)indx[j] * k;
          if (tkern == 'g')
             for (IT t = 0; t < k; t++) ci[t] += bj[t];
          else if (tkern == 'm')
             for (IT t = 0; t < k; t++) ci[t] += val[j] * bj[t];
          else if (tkern == 's')
          {
-            float s = 0;
+            VT s = 0;
             for (IT t = 0; t < k; t++) s += ai[t] * bj[t];
-            float d = table_sigmoid(s);
-            for (IT t = 0; t < k; t++) ci[t] = (float)(ci[t] + (1.0 - d) * bj[t]);
+            VT d = table_sigmoid(s);
+            for (IT t = 0; t < k; t++) ci[t] = (VT)(ci[t] + (1.0 - d) * bj[t]);
          }
          else
          {
-            float s = 0;
+            VT s = 0;
             for (IT t = 0; t < k; t++)
             {
                T[t] = ai[t] - bj[t];
                s += T[t] * T[t];
             }
-            float d;
+            VT d;
             if (tkern == 't')
             {
-               d = (float)(-2.0 / (1.0 + s));
-               d = d > 5.0f ? 5.0f : (d < -5.0f ? -5.0f : d);
+               d = (VT)(-2.0 / (1.0 + s));
+               d = d > (VT)5.0 ? (VT)5.0 : (d < (VT)-5.0 ? (VT)-5.0 : d);
             }
             else
-               d = (float)(1.0 + 1.0 / s);
+               d = (VT)(1.0 + 1.0 / s);
             for (IT t = 0; t < k; t++) ci[t] = ci[t] + d * T[t];
          }
       }
@@ -157,7 +163,7 @@ static double flops_per_edge(char tkern, IT k)
 }
 static double algorithmic_bytes(char tkern, IT m, IT k, int64_t nnz)
 {
-   const double F = 4, I = sizeof(IT);
+   const double F = sizeof(VT), I = sizeof(IT);
    const double vb = tkern == 'm' ? F : 0, xb = (tkern == 's' || tkern == 't' || tkern == 'f') ? F * k : 0;
    return nnz * (F * k + I + vb) + (double)m * (xb + F * k + 2 * I);
 }
@@ -210,7 +216,7 @@ int main(int narg, char **argv)
    }
    if (inputfile.empty()) { printf("Need input file ??? \n"); return 1; }
    if (!strchr("tfsmg", tkern)) { printf("unknown kernel kind '%c'\n", tkern); return 1; }
-   const float alpha = 1.0f, beta = ibeta == 0 ? 0.0f : 1.0f;
+   const VT alpha = 1.0, beta = ibeta == 0 ? 0.0 : 1.0;
    if (nrep < 1) nrep = 1;
 
    fmm_host::CsrMatrix<IT> S;
@@ -228,9 +234,9 @@ int main(int narg, char **argv)
 
    // inputs as the reference's tester draws them
    std::default_random_engine gen;
-   std::uniform_real_distribution<float> dist(0.0f, 1.0f);
+   std::uniform_real_distribution<VT> dist(0.0, 1.0);
    const size_t szA = (size_t)M * K, szB = (size_t)N * K, szC = (size_t)M * K;
-   std::vector<float> a(szA), b(szB), c(szC, 0.0f), c0(szC, 0.0f), values((size_t)S.nnz);
+   std::vector<VT> a(szA), b(szB), c(szC, (VT)0), c0(szC, (VT)0), values((size_t)S.nnz);
    for (auto &v : a) v = dist(gen);
    for (auto &v : b) v = dist(gen);
    for (auto &v : values) v = dist(gen);
@@ -250,7 +256,7 @@ int main(int narg, char **argv)
       if (rc) { fprintf(stderr, "fusedMM_csr returned %d\n", rc); return 1; }
       // bound of the reference's checker (:816-831) with the true maximum degree:
       // 2 * Md * flops-per-element * eps; the sigmoid table adds one bin of slack per edge
-      const double eps = 5.9604644775390625e-08 * 2;
+      const double eps = sizeof(VT) == 4 ? 1.1920928955078125e-07 : 2.220446049250313e-16;
       double per = (tkern == 's') ? (4.0 * K + 6) : (tkern == 'm') ? 2.0 * K : (tkern == 'g') ? 1.0 * K : (5.0 * K + 2);
       double bound = 2.0 * (double)maxdeg * per * eps;
       if (tkern == 's') bound += 1.3e-3 * std::sqrt((double)maxdeg);
@@ -267,8 +273,8 @@ int main(int narg, char **argv)
       }
       if (nerr) { printf("FAILED TEST, %lld ELEMENTS!!!\n", (long long)nerr); return 1; }
       printf("PASSED TEST\n");
-      std::fill(c.begin(), c.end(), 0.0f);
-      std::fill(c0.begin(), c0.end(), 0.0f);
+      std::fill(c.begin(), c.end(), (VT)0);
+      std::fill(c0.begin(), c0.end(), (VT)0);
    }
 
    // ---- trusted timing (CPU) -------------------------------------------------------------
@@ -288,25 +294,25 @@ int main(int narg, char **argv)
    if (use_gpu_resident)
    {
       // working-set rotation: enough copies to exceed the cache size asked for
-      const double ws = 4.0 * (szA + szB + szC + (double)S.nnz) + sizeof(IT) * ((double)S.nnz + 2.0 * (M + 1));
+      const double ws = (double)sizeof(VT) * (szA + szB + szC + (double)S.nnz) + sizeof(IT) * ((double)S.nnz + 2.0 * (M + 1));
       int ncopies = 1;
       if (csKB > 0 && ws < 1024.0 * csKB) ncopies = (int)std::ceil(1024.0 * csKB / ws);
-      struct Dev { float *a, *b, *c, *val; IT *idx, *ptr; };
+      struct Dev { VT *a, *b, *c, *val; IT *idx, *ptr; };
       std::vector<Dev> d((size_t)ncopies);
       {
          Range r("h2d");
          for (auto &x : d)
          {
-            HIP_OK(hipMalloc((void **)&x.a, szA * 4));
-            HIP_OK(hipMalloc((void **)&x.b, szB * 4));
-            HIP_OK(hipMalloc((void **)&x.c, szC * 4));
-            HIP_OK(hipMalloc((void **)&x.val, std::max<size_t>(1, (size_t)S.nnz) * 4));
+            HIP_OK(hipMalloc((void **)&x.a, szA * sizeof(VT)));
+            HIP_OK(hipMalloc((void **)&x.b, szB * sizeof(VT)));
+            HIP_OK(hipMalloc((void **)&x.c, szC * sizeof(VT)));
+            HIP_OK(hipMalloc((void **)&x.val, std::max<size_t>(1, (size_t)S.nnz) * sizeof(VT)));
             HIP_OK(hipMalloc((void **)&x.idx, std::max<size_t>(1, (size_t)S.nnz) * sizeof(IT)));
             HIP_OK(hipMalloc((void **)&x.ptr, ((size_t)S.rows + 1) * sizeof(IT)));   // rows + 1 pointers
-            HIP_OK(hipMemcpy(x.a, a.data(), szA * 4, hipMemcpyHostToDevice));
-            HIP_OK(hipMemcpy(x.b, b.data(), szB * 4, hipMemcpyHostToDevice));
-            HIP_OK(hipMemset(x.c, 0, szC * 4));
-            HIP_OK(hipMemcpy(x.val, values.data(), (size_t)S.nnz * 4, hipMemcpyHostToDevice));
+            HIP_OK(hipMemcpy(x.a, a.data(), szA * sizeof(VT), hipMemcpyHostToDevice));
+            HIP_OK(hipMemcpy(x.b, b.data(), szB * sizeof(VT), hipMemcpyHostToDevice));
+            HIP_OK(hipMemset(x.c, 0, szC * sizeof(VT)));
+            HIP_OK(hipMemcpy(x.val, values.data(), (size_t)S.nnz * sizeof(VT), hipMemcpyHostToDevice));
             HIP_OK(hipMemcpy(x.idx, S.colids.data(), (size_t)S.nnz * sizeof(IT), hipMemcpyHostToDevice));
             HIP_OK(hipMemcpy(x.ptr, S.rowptr.data(), ((size_t)S.rows + 1) * sizeof(IT), hipMemcpyHostToDevice));
          }

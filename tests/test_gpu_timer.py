@@ -49,3 +49,27 @@ def test_reference_style_c_caller(bits):
     and passes host arrays -- the reference's calling convention, untouched."""
     r = subprocess.run([fbuild.dropin_path(bits)], stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True, timeout=110)
     assert r.returncode == 0 and "PASSED" in r.stdout, r.stdout
+
+
+def test_timer_double_precision(tmp_path):
+    g = synth.er_graph(2048, 16384, 3, 64)
+    path = str(tmp_path / "er.mtx")
+    synth.write_mtx_symmetric(path, g)
+    for tkern in ("s", "t", "m"):
+        r = subprocess.run([fbuild.timer_path(64, 64), "-input", path, "-T", "1", "-K", "96", "-t", tkern, "-nrep", "2"],
+                           stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True, timeout=110)
+        assert r.returncode == 0 and "PASSED TEST" in r.stdout, r.stdout
+
+
+def test_sweep_script(tmp_path):
+    """The counterpart of the reference's runtime.sh: one CSV per dataset and kind."""
+    g = synth.er_graph(1024, 8192, 4, 32)
+    path = str(tmp_path / "tiny.mtx")
+    synth.write_mtx_symmetric(path, g)
+    script = os.path.join(os.path.dirname(fbuild.timer_path(32)), "..", "runtime_sweep.sh")
+    r = subprocess.run(["bash", script, "-i", "32", "-r", str(tmp_path / "res"), path],
+                       stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True, timeout=280)
+    assert r.returncode == 0, r.stdout
+    lines = open(str(tmp_path / "res" / "tiny-s-sreal-gpu.csv")).read().strip().splitlines()
+    assert lines[0].startswith("Filename,NNZ") and len(lines) == 9
+    assert [l.split(",")[4] for l in lines[1:]] == ["32", "64", "96", "128", "160", "192", "224", "256"]
