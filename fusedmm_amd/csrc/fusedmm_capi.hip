@@ -85,6 +85,7 @@ struct Globals {
    int64_t heavy_deg = 0;
    int seg_len = 0;
    int blocks_per_cu = 0;
+   int validate = 0;
    fusedMM_amd_sop_fn sop_fn = nullptr;
    bool timing = false;
    int timing_calls = 0;
@@ -113,6 +114,7 @@ void read_env_once()
    g.sop_kind_from_env_done = true;
    if (const char *e = getenv("FUSEDMM_SOP_KIND")) g.sop_kind = sop_kind_from_name(e);
    if (const char *e = getenv("FUSEDMM_BLOCKS_PER_CU")) g.blocks_per_cu = atoi(e);
+   if (const char *e = getenv("FUSEDMM_VALIDATE")) g.validate = atoi(e);
 }
 
 // The 2048-entry sigmoid table, built with the expressions of the reference's
@@ -563,6 +565,38 @@ int edge_scalars(const Args &a, val_t *d_s, DeviceState *d, hipStream_t stream)
    return FUSEDMM_SUCCESS_RETURN;
 }
 
+// FUSEDMM_VALIDATE=1 / fusedMM_amd_set_validate(1): check row pointers and
+// column ids on the device before any kernel dereferences them.  Costs a pass
+// over the CSR arrays and a synchronisation per call.
+int validate_operands(const Args &a, hipStream_t stream)
+{
+   if (a.n <= 0 || !a.indx || !a.pntrb || !a.pntre)
+   {
+      FMM_LOG("operand check: n must be positive and the CSR arrays non-NULL");
+      return FUSEDMM_FAIL_RETURN;
+   }
+   DeviceState *d = nullptr;
+   int st = device_state(&d);
+   if (st) return st;
+   Params<idx_t> p;
+   memset(&p, 0, sizeof(p));
+   p.pntrb = a.pntrb; p.pntre = a.pntre; p.indx = a.indx; p.m = a.m;
+   unsigned int *flag = &d->ctr->invalid;
+   FMM_HIP(hipMemsetAsync(flag, 0, sizeof(unsigned int), stream));
+   int64_t blocks = (a.m + kWavesPerBlock - 1) / kWavesPerBlock;
+   if (blocks > (int64_t)d->num_cu * 8) blocks = (int64_t)d->num_cu * 8;
+   hipLaunchKernelGGL(validate_kernel<idx_t>, dim3((unsigned int)blocks), dim3(kBlockThreads), 0, stream, p, a.n, flag);
+   unsigned int h = 0;
+   FMM_HIP(hipMemcpyAsync(&h, flag, sizeof(h), hipMemcpyDeviceToHost, stream));
+   FMM_HIP(hipStreamSynchronize(stream));
+   if (h)
+   {
+      FMM_LOG("operand check failed: a column id outside [0, n) or a row with pntre < pntrb");
+      return FUSEDMM_FAIL_RETURN;
+   }
+   return FUSEDMM_SUCCESS_RETURN;
+}
+
 int64_t max_slot(const idx_t *h_pe, int64_t m)
 {
    int64_t slots = 0;
@@ -623,6 +657,11 @@ int run_wide_reduction(const Args &a, const Plan &pl, int sop_kind)
 int run_on_device(const Args &a, const Plan &pl, int sop_kind, hipStream_t stream)
 {
    if (a.m <= 0 || a.k < 1) return FUSEDMM_SUCCESS_RETURN;
+   if (g.validate)
+   {
+      int st = validate_operands(a, stream);
+      if (st) return st;
+   }
    if (a.k <= kMaxK) return run_slab(a, pl, sop_kind, stream);
    if (a.ldy < a.k || a.ldz < a.k || (pl.reads_x && a.ldx < a.k))
    {
@@ -847,6 +886,15 @@ int fusedMM_amd_set_opt(int enable)
    std::lock_guard<std::mutex> lock(g.mu);
    int prev = g.opt;
    g.opt = enable ? 1 : 0;
+   return prev;
+}
+
+int fusedMM_amd_set_validate(int enable)
+{
+   std::lock_guard<std::mutex> lock(g.mu);
+   read_env_once();
+   int prev = g.validate;
+   g.validate = enable ? 1 : 0;
    return prev;
 }
 

@@ -55,7 +55,7 @@ struct Counters {
    unsigned int n_heavy;    // heavy rows queued by the row kernel
    unsigned int n_seg;      // edge segments queued
    unsigned int overflow;   // heavy rows that did not fit the queue (handled inline)
-   unsigned int pad;
+   unsigned int invalid;    // set by the optional operand check
    unsigned int pad2[28];         // keep the row counters on their own 128-byte lines
    // Row claim counters.  Read-modify-writes on ONE address retire one per
    // ~12 ns on this GPU however many CUs issue them; on distinct 128-byte
@@ -997,6 +997,29 @@ __global__ __launch_bounds__(kBlockThreads) void apply_sop_kernel(real_t *s, int
 {
    for (int64_t i = (int64_t)blockIdx.x * kBlockThreads + threadIdx.x; i < n; i += (int64_t)gridDim.x * kBlockThreads)
       s[i] = sop_eval(sop_kind, s[i], tab);
+}
+
+// Optional operand check (off by default, like the reference, which trusts its
+// caller): a column id outside [0, n) or a row with pntre < pntrb would make the
+// kernels read outside Y.  Sets flag[0] when anything is wrong.
+template <typename IdxT>
+__global__ __launch_bounds__(kBlockThreads) void validate_kernel(const Params<IdxT> p, int64_t n, unsigned int *flag)
+{
+   const int lane = threadIdx.x & 63;
+   const int64_t wave0 = (int64_t)blockIdx.x * kWavesPerBlock + (threadIdx.x >> 6);
+   const int64_t nwaves = (int64_t)gridDim.x * kWavesPerBlock;
+   bool bad = false;
+   for (int64_t row = wave0; row < p.m; row += nwaves)
+   {
+      const IdxT jb = p.pntrb[row], je = p.pntre[row];
+      if (je < jb || jb < 0) { bad = true; continue; }
+      for (IdxT j = jb + lane; j < je; j += 64)
+      {
+         const IdxT c = p.indx[j];
+         if (c < 0 || (int64_t)c >= n) bad = true;
+      }
+   }
+   if (bad) atomicOr(flag, 1u);
 }
 
 // Clears the queue and claim counters before each call.  A kernel rather than a

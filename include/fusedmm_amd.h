@@ -99,6 +99,14 @@ int fusedMM_amd_value_bytes(void);
  * the previous setting. */
 int fusedMM_amd_set_opt(int enable);
 
+/* 1: before each call, check on the device that every row has pntrb <= pntre
+ * and every column id lies in [0, n); a call with bad operands then returns
+ * FUSEDMM_FAIL_RETURN instead of reading outside Y.  Off by default (the
+ * reference does not check either); also enabled by FUSEDMM_VALIDATE=1.
+ * Costs one pass over the CSR arrays and a synchronisation.  Returns the
+ * previous setting. */
+int fusedMM_amd_set_validate(int enable);
+
 /* Tuning knobs of the heavy-row split: rows with more than `heavy_deg` edges
  * are cut into segments of `seg_len` edges (0, 0 restores the K-dependent
  * defaults).  For tests and experiments. */

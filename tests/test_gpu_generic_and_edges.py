@@ -228,3 +228,30 @@ def test_stream_entry_can_be_captured_in_a_hip_graph(oracle):
         rc = fa.fusedMM_csr(fa.MSG_SIGMOID, g["rows"], g["cols"], k, 1.0, g["nnz"], g["rows"], g["cols"], val, indx,
                             pb, pe, dX, k, dY2, k, 0.0, Ze2, k)
         assert rc == 0
+
+
+def test_operand_check_rejects_bad_csr_instead_of_reading_outside_y():
+    """With the optional check on, a column id >= n or a row with pntre < pntrb
+    returns FUSEDMM_FAIL_RETURN before any kernel dereferences it."""
+    lib = fa.load(32)
+    prev = lib.fusedMM_amd_set_validate(1)
+    try:
+        g = graphs.tiny_er(50, 120, 2)
+        k = 32
+        Y = graphs.features(50, k, 2)
+        Z0 = np.zeros((50, k), np.float32)
+        rc, _ = gpu_api.run(MSG["g"], g, None, Y, Z0)
+        assert rc == 0                                   # clean operands pass
+        bad = dict(g)
+        bad["indx"] = g["indx"].copy()
+        bad["indx"][7] = 50                              # one past the last row of Y
+        for where in ("device", "host"):
+            rc, Z = gpu_api.run(MSG["g"], bad, None, Y, Z0, where=where)
+            assert rc == fa.FAIL and not Z.any()
+        bad = dict(g)
+        bad["pntre"] = g["pntre"].copy()
+        bad["pntre"][3] = g["pntrb"][3] - 1
+        rc, _ = gpu_api.run(MSG["g"], bad, None, Y, Z0)
+        assert rc == fa.FAIL
+    finally:
+        lib.fusedMM_amd_set_validate(prev)
