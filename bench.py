@@ -24,9 +24,9 @@ PEAK_HBM_GBPS = 8000.0
 
 # HBM bytes per launch of the dominant kernel from rocprofv3 --pmc FETCH_SIZE and
 # WRITE_SIZE, each scaled by the same counter's reading for a plain 1 GiB copy
-# (profiles/rows_kernel_sigmoid_k128_c2.md, profiles/spmm_k256_c3_rmat22.md).  Measured, not computed: refreshed
+# (one summary per workload under profiles/).  Measured, not computed: refreshed
 # whenever the kernel changes.
-MEASURED_TRAFFIC_BYTES = {"c2": 9789942792, "c3": 127814327894}
+MEASURED_TRAFFIC_BYTES = {"c2": 9789942792, "c3": 127814327894, "c4": 129555164044, "c5": 91009602274}
 
 WORKLOADS = {
     # name: (description, op letter, K, sop kind)
