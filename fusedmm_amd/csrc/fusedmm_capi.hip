@@ -481,9 +481,8 @@ int stage_up(const Args &h, const Plan &pl, Args *a, int64_t *slots_out)
    if (pl.reads_x) FMM_HIP(hipMemcpyAsync(d->stage[4].ptr, h.x, b_x, hipMemcpyHostToDevice, s));
    FMM_HIP(hipMemcpyAsync(d->stage[5].ptr, h.y, b_y, hipMemcpyHostToDevice, s));
    const bool overwrite = pl.opt_rule && h.beta == 0.0f;
-   if (!overwrite)
-      FMM_HIP(hipMemcpy2DAsync(d->stage[6].ptr, (size_t)h.ldz * kValBytes, h.z, (size_t)h.ldz * kValBytes, (size_t)h.k * kValBytes, (size_t)h.m,
-                               hipMemcpyHostToDevice, s));
+   if (!overwrite)   // one contiguous copy, padding columns included (they are never written back)
+      FMM_HIP(hipMemcpyAsync(d->stage[6].ptr, h.z, b_z - (size_t)(h.ldz - h.k) * kValBytes, hipMemcpyHostToDevice, s));
    *a = h;
    a->pntrb = (const idx_t *)d->stage[0].ptr;
    a->pntre = (const idx_t *)d->stage[1].ptr;
@@ -498,12 +497,24 @@ int stage_up(const Args &h, const Plan &pl, Args *a, int64_t *slots_out)
 }
 
 // Only the first k columns of each Z row are written back, as the reference
-// touches nothing else.
+// touches nothing else.  With ldz == k that is one contiguous copy; otherwise
+// the block is fetched contiguously and the k columns of every row are copied
+// out on the host (a strided device copy of millions of short rows is far
+// slower than either).
 int stage_down(const Args &h, const Args &a)
 {
-   FMM_HIP(hipMemcpy2DAsync(h.z, (size_t)h.ldz * kValBytes, a.z, (size_t)h.ldz * kValBytes, (size_t)h.k * kValBytes, (size_t)h.m,
-                            hipMemcpyDeviceToHost, 0));
+   const size_t span = ((size_t)h.m * (size_t)h.ldz - (size_t)(h.ldz - h.k)) * kValBytes;
+   if (h.ldz == h.k)
+   {
+      FMM_HIP(hipMemcpyAsync(h.z, a.z, span, hipMemcpyDeviceToHost, 0));
+      FMM_HIP(hipStreamSynchronize(0));
+      return FUSEDMM_SUCCESS_RETURN;
+   }
+   std::vector<val_t> tmp(span / kValBytes);
+   FMM_HIP(hipMemcpyAsync(tmp.data(), a.z, span, hipMemcpyDeviceToHost, 0));
    FMM_HIP(hipStreamSynchronize(0));
+   for (int64_t i = 0; i < h.m; i++)
+      memcpy(h.z + i * h.ldz, tmp.data() + i * h.ldz, (size_t)h.k * kValBytes);
    return FUSEDMM_SUCCESS_RETURN;
 }
 
@@ -635,7 +646,7 @@ int run_wide_reduction(const Args &a, const Plan &pl, int sop_kind)
    FMM_HIP(hipMemcpy(he.data(), a.pntre, (size_t)a.m * sizeof(idx_t), hipMemcpyDeviceToHost));
    const int64_t slots = max_slot(he.data(), a.m);
    if (pl.opt_rule && a.beta == 0.0f)
-      FMM_HIP(hipMemset2DAsync(a.z, (size_t)a.ldz * kValBytes, 0, (size_t)a.k * kValBytes, (size_t)a.m, 0));
+      hipLaunchKernelGGL(zero_rows_kernel, dim3((unsigned int)(d->num_cu * 8)), dim3(kBlockThreads), 0, 0, a.z, a.m, a.k, a.ldz);
    if (slots <= 0) return FUSEDMM_SUCCESS_RETURN;
    st = grow(d->stage[7], (size_t)slots * kValBytes);
    if (st) return st;
@@ -700,7 +711,7 @@ int run_host_sop(const Args &a, const idx_t *h_pb, const idx_t *h_pe, int64_t sl
    if (st) return st;
    const bool overwrite = pl.opt_rule && a.beta == 0.0f;
    if (overwrite)
-      FMM_HIP(hipMemset2DAsync(a.z, (size_t)a.ldz * kValBytes, 0, (size_t)a.k * kValBytes, (size_t)a.m, 0));
+      hipLaunchKernelGGL(zero_rows_kernel, dim3((unsigned int)(d->num_cu * 8)), dim3(kBlockThreads), 0, 0, a.z, a.m, a.k, a.ldz);
    if (slots <= 0) return hip_status(hipStreamSynchronize(0), "hipStreamSynchronize");
    st = grow(d->stage[7], (size_t)slots * kValBytes);
    if (st) return st;

@@ -1022,6 +1022,15 @@ __global__ __launch_bounds__(kBlockThreads) void validate_kernel(const Params<Id
    if (bad) atomicOr(flag, 1u);
 }
 
+// Z[i, 0:k] = 0 for i < m (the overwrite rule of the pattern tuples, when the
+// accumulate pass that follows can only add).
+__global__ __launch_bounds__(kBlockThreads) void zero_rows_kernel(real_t *z, int64_t m, int64_t k, int64_t ldz)
+{
+   const int64_t total = m * k;
+   for (int64_t i = (int64_t)blockIdx.x * kBlockThreads + threadIdx.x; i < total; i += (int64_t)gridDim.x * kBlockThreads)
+      z[(i / k) * ldz + (i % k)] = (real_t)0;
+}
+
 // Clears the queue and claim counters before each call.  A kernel rather than a
 // memset so that callers may capture the stream entry point in a HIP graph.
 __global__ __launch_bounds__(kBlockThreads) void reset_counters_kernel(Counters *c)
