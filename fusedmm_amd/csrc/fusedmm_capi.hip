@@ -446,6 +446,27 @@ bool is_device_pointer(const void *p)
    return attr.type == hipMemoryTypeDevice || attr.type == hipMemoryTypeManaged;
 }
 
+// The synchronous entry point takes operands that are all host memory or all
+// device memory.  Returns 1 (device), 0 (host) or -1 (mixed: refused, a kernel
+// dereferencing a host address would fault the GPU).
+int operand_residence(const Args &a)
+{
+   const void *ops[] = {a.z, a.y, a.x, a.val, a.indx, a.pntrb, a.pntre};
+   int dev = 0, host = 0;
+   for (const void *o : ops)
+   {
+      if (!o) continue;
+      if (is_device_pointer(o)) dev++;
+      else host++;
+   }
+   if (dev && host)
+   {
+      FMM_LOG("operands mix host and device memory; pass all of one kind");
+      return -1;
+   }
+   return dev ? 1 : 0;
+}
+
 // Host-pointer mode: copy the operands to the GPU.  On return `a` holds device
 // addresses and `slots` is one past the last edge slot any processed row uses.
 int stage_up(const Args &h, const Plan &pl, Args *a, int64_t *slots_out)
@@ -783,7 +804,9 @@ int entry(const Args &a, bool async, hipStream_t stream)
             return FUSEDMM_UNDEFINED_USER_FUNCTION;
          }
          if (a.m <= 0 || a.k < 1) return FUSEDMM_SUCCESS_RETURN;
-         if (is_device_pointer(a.z))
+         const int where = operand_residence(a);
+         if (where < 0) return FUSEDMM_FAIL_RETURN;
+         if (where == 1)
          {
             std::vector<idx_t> hb((size_t)a.m), he((size_t)a.m);
             FMM_HIP(hipMemcpy(hb.data(), a.pntrb, (size_t)a.m * sizeof(idx_t), hipMemcpyDeviceToHost));
@@ -802,7 +825,10 @@ int entry(const Args &a, bool async, hipStream_t stream)
       }
    }
    if (async) return run_on_device(a, pl, sop_kind, stream);
-   if (is_device_pointer(a.z))
+   if (a.m <= 0 || a.k < 1) return FUSEDMM_SUCCESS_RETURN;
+   const int where = operand_residence(a);
+   if (where < 0) return FUSEDMM_FAIL_RETURN;
+   if (where == 1)
    {
       st = run_on_device(a, pl, sop_kind, 0);
       if (st) return st;

@@ -255,3 +255,17 @@ def test_operand_check_rejects_bad_csr_instead_of_reading_outside_y():
         assert rc == fa.FAIL
     finally:
         lib.fusedMM_amd_set_validate(prev)
+
+
+def test_mixed_host_and_device_operands_are_refused():
+    import torch
+    g = graphs.tiny_er(50, 120, 2)
+    k = 32
+    Y = graphs.features(50, k, 2)
+    dev = torch.device("cuda:0")
+    Zd = torch.zeros((50, k), device=dev)
+    rc = fa.fusedMM_csr(fa.MSG_GCN, 50, 50, k, 1.0, g["nnz"], 50, 50, g["val"], g["indx"], np.ascontiguousarray(g["pntrb"]),
+                        np.ascontiguousarray(g["pntre"]), None, k, Y, k, 0.0, Zd, k)       # Z on the GPU, the rest on the host
+    assert rc == fa.FAIL
+    torch.cuda.synchronize()
+    assert not Zd.any()
