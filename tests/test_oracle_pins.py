@@ -263,3 +263,48 @@ def test_gpu_bin_expression_is_equivalent_for_every_float(oracle):
     bad = oracle.lib.orc_count_bin_formula_mismatches(C.byref(seen))
     assert seen.value == 2168455170
     assert bad == 0
+
+
+def test_partition_hand_example_and_properties(oracle):
+    """nnz-balanced contiguous row ranges (reference fusedMM.c:633-676).  The row
+    that tips the running count over the quota OPENS the next thread's range."""
+    deg = np.array([3, 1, 1, 1, 3, 1], np.int32)
+    ptr = np.concatenate([[0], np.cumsum(deg)]).astype(np.int32)
+    rc, rb, re = oracle.partition(ptr[:-1], ptr[1:], 2)
+    # Mnnz = 10, quota 5: running counts 3,4,5,6 -> row 3 is the first to exceed it
+    assert rc == 0 and rb.tolist() == [0, 3] and re.tolist() == [3, 6]
+    # three threads: quota 3; row 1 tips (4 > 3) -> thread 1 starts at 1 with quota (10-4)/2 = 3;
+    # running 1,2,5 -> row 4 tips -> thread 2 starts at 4
+    rc, rb, re = oracle.partition(ptr[:-1], ptr[1:], 3)
+    assert rb.tolist() == [0, 1, 4] and re.tolist() == [1, 4, 6]
+    # properties on random skewed degrees: ranges tile [0, m) in order, nobody is far over the mean
+    rng = np.random.default_rng(1)
+    for nthreads in (2, 7, 16):
+        deg = np.minimum(rng.zipf(1.6, 5000), 400).astype(np.int64)
+        ptr = np.concatenate([[0], np.cumsum(deg)]).astype(np.int64)
+        rc, rb, re = oracle.partition(ptr[:-1], ptr[1:], nthreads)
+        assert rc == 0 and rb[0] == 0
+        used = [(b, e) for b, e in zip(rb, re) if e >= 0]
+        assert used[-1][1] == 5000
+        for (b0, e0), (b1, e1) in zip(used, used[1:]):
+            assert e0 == b1 and b0 <= e0
+        loads = [int(ptr[e] - ptr[b]) for b, e in used]
+        assert max(loads) <= ptr[-1] / nthreads + 2 * 400 + ptr[-1] / nthreads * 0.5
+
+
+@pytest.mark.parametrize("t,sk", [("s", SOP_SIGMOID), ("t", SOP_TDIST), ("m", 0), ("g", 0)])
+def test_cpu_baseline_agrees_with_the_fp64_evaluation(t, sk):
+    """The function bench.py times as its CPU leg (vectorised, thread-partitioned)."""
+    from oracle_api import Oracle
+    fast, ref = Oracle(fast=True), Oracle()
+    g = graphs.with_values(graphs.tiny_er(500, 4000, 9))
+    k = 64
+    X = graphs.features(500, k, 1, -0.3, 0.3, 1)
+    Y = graphs.features(500, k, 1, -0.3, 0.3, 2)
+    for threads in (1, 3, 8):
+        Z = graphs.features(500, k, 1, -1, 1, 3)
+        assert fast.baseline(t, g, X, Y, Z, 0.0, sk, threads) == 0
+        want = np.zeros((500, k), np.float32)
+        ref.opt(t, g, X, Y, want, beta=0.0, sop_kind=sk, mode=1)
+        tol = 2e-3 if t == "s" else 2e-5              # sigmoid: a table-bin flip between summation orders
+        np.testing.assert_allclose(Z, want, rtol=tol, atol=tol)
