@@ -5,9 +5,11 @@
  * check and the CPU-baseline leg of the benchmark may load it; the shipped
  * library never links, loads or calls anything in this directory.
  *
- * Each function names the reference file:line it restates.  Index-width
- * dependent functions live in fusedmm_oracle_body.inc and are compiled twice
- * (suffix _i32 / _i64), mirroring the reference's compile-time INDEXTYPE.
+ * Each function names the reference file:line it restates.  Value-type
+ * dependent functions live in fusedmm_oracle_val.inc (float: no suffix, double:
+ * _d), index-width dependent ones in fusedmm_oracle_body.inc (suffixes _i32,
+ * _i64, _d_i32, _d_i64), mirroring the reference's compile-time INDEXTYPE and
+ * SREAL / DREAL.  Every pin below holds for both precisions.
  *
  * Pinning status (what independently checks each function):
  *   orc_sigmoid_table / orc_sigmoid_lookup / orc_sop
@@ -20,8 +22,10 @@
  *          inputs; scipy CSR @ Y for the spmm/gcn tuples; dense brute force.
  *   orc_fusedmm_opt_*      - golden Z from the reference harness's trusted
  *          kernels and generic fusedMM_csr; dense fp64 brute force; invariants.
- *   orc_partition_rows_*   - brute-force property check (ranges tile [0,m),
- *          boundaries follow the running-quota rule) and golden vectors.
+ *   orc_partition_rows_*   - hand-computed examples and properties (ranges tile
+ *          [0,m) in order, bounded imbalance).  The reference does not expose its
+ *          partition, so no vector of its own pins this one: PARITY UNPINNED
+ *          beyond those checks.  Only the CPU baseline's thread ranges use it.
  *   orc_gpu_dot / mode 2   - equals the fp64 dot within K*eps*sum|x*y|; equals
  *          the sequential dot exactly for inputs whose products are exactly
  *          representable (small integers), which a wrong lane map would break.
