@@ -115,6 +115,12 @@ void read_env_once()
    if (const char *e = getenv("FUSEDMM_SOP_KIND")) g.sop_kind = sop_kind_from_name(e);
    if (const char *e = getenv("FUSEDMM_BLOCKS_PER_CU")) g.blocks_per_cu = atoi(e);
    if (const char *e = getenv("FUSEDMM_VALIDATE")) g.validate = atoi(e);
+   if (const char *e = getenv("FUSEDMM_SPLIT"))   // "heavy_deg,seg_len", as fusedMM_amd_set_split
+   {
+      long long h = 0;
+      int sl = 0;
+      if (sscanf(e, "%lld,%d", &h, &sl) == 2 && h > 0 && sl > 0) { g.heavy_deg = h; g.seg_len = sl; }
+   }
 }
 
 // The 2048-entry sigmoid table, built with the expressions of the reference's
@@ -370,8 +376,10 @@ int run_slab(const Args &a, const Plan &pl, int sop_kind, hipStream_t stream)
    p.imessage = a.imessage;
    p.sigmoid_table = d->sigmoid_table;
 
-   // heavy-row split: segments of about 256 KiB of gathered rows
-   int seg_len = g.seg_len > 0 ? g.seg_len : (int)(262144 / ((int64_t)kValBytes * a.k));
+   // heavy-row split: segments of about 1 MiB of gathered rows (measured best on the
+   // R-MAT and power-law benchmark graphs: shorter segments pay their start-up and
+   // partial-result cost more often, longer ones leave long rows to single waves)
+   int seg_len = g.seg_len > 0 ? g.seg_len : (int)(1048576 / ((int64_t)kValBytes * a.k));
    if (seg_len < 64 && g.seg_len <= 0) seg_len = 64;
    int64_t heavy_deg = g.heavy_deg > 0 ? g.heavy_deg : 2 * (int64_t)seg_len;
    if (heavy_deg < seg_len) heavy_deg = seg_len;

@@ -72,9 +72,10 @@ struct HeavyRow {
 };
 
 struct SegDesc {
-   int64_t row;
-   unsigned int seg;       // segment number inside the row
-   unsigned int len;       // edges per segment of this row
+   int64_t row;            // -1: slot of a row that did not fit the queue
+   int64_t first;          // first edge slot of the segment
+   unsigned int count;     // edges in the segment
+   unsigned int pad;
 };
 
 constexpr int kRowsPerClaim = 8;        // rows a wave claims at a time
@@ -595,23 +596,28 @@ __device__ __forceinline__ double chunk_entry(double v, int e)
 // Edges [jb, je) of one row, dealt round-robin to the sub-waves.  Column ids
 // (and edge values) are fetched 64 at a time with one coalesced load per
 // array, the next 64 while the current ones are being used; U gathers are in
-// flight per sub-wave.  All lanes of the wave call this with the same jb, je.
+// flight per sub-wave.  All lanes of the wave call this with the same arguments.
 template <int V, int L, int R, bool EXACT, int OP, int SOPK, int U, typename IdxT>
 __device__ __forceinline__ void walk_edges(Slice<R> &acc, const Slice<R> &xs, const Params<IdxT> &p,
-                                           IdxT jb, IdxT je, int lane, const real_t *tab)
+                                           IdxT jb, IdxT je, EdgeChunk<IdxT> &cur, IdxT next_b, IdxT next_e, int lane,
+                                           const real_t *tab)
 {
    constexpr int S = 64 / L;
    const int sub = (L == 64) ? 0 : lane / L, sl = (L == 64) ? lane : lane % L;
    const int sop_kind = SOPK >= 0 ? SOPK : p.sop_kind;
-   if (jb >= je) return;
-   EdgeChunk<IdxT> cur;
-   load_chunk<OP, IdxT>(cur, p, jb, je, lane);
+   // On entry `cur` holds slots [jb, jb+64) (requested by the caller); on exit it
+   // holds slots [next_b, next_b+64) of whatever the caller walks next, requested
+   // while the last chunk of this row was being gathered.
+   if (jb >= je)
+   {
+      load_chunk<OP, IdxT>(cur, p, next_b, next_e, lane);
+      return;
+   }
    for (IdxT j0 = jb; j0 < je; j0 += 64)
    {
       EdgeChunk<IdxT> nxt;
-      nxt.col = 0;
-      nxt.val = (real_t)0;
       if (j0 + 64 < je) load_chunk<OP, IdxT>(nxt, p, j0 + 64, je, lane);
+      else load_chunk<OP, IdxT>(nxt, p, next_b, next_e, lane);
       const int n = (je - j0) < 64 ? (int)(je - j0) : 64;
       for (int b0 = 0; b0 < n; b0 += S * U)
       {
@@ -777,7 +783,12 @@ __global__ __launch_bounds__(kBlockThreads) void rows_kernel(const Params<IdxT> 
          if (fits)
          {
             if (lane == 0) p.heavy[slot] = HeavyRow{row, base, nseg};
-            for (unsigned int s = lane; s < nseg; s += 64) p.segs[base + s] = SegDesc{row, s, (unsigned int)seg_len};
+            for (unsigned int s = lane; s < nseg; s += 64)
+            {
+               const int64_t off = (int64_t)s * seg_len;
+               const int64_t cnt = deg - off < seg_len ? deg - off : seg_len;
+               p.segs[base + s] = SegDesc{row, (int64_t)jb + off, (unsigned int)cnt, 0u};
+            }
             continue;
          }
          // mark the slot unused (the merge kernel skips n_seg == 0) and do the row here
@@ -788,7 +799,7 @@ __global__ __launch_bounds__(kBlockThreads) void rows_kernel(const Params<IdxT> 
          }
          // every queue entry below the cap has exactly one writer: poison ours
          for (uint64_t s = (uint64_t)base + lane; s < (uint64_t)base + nseg && s < (uint64_t)p.cap_seg; s += 64)
-            p.segs[s] = SegDesc{-1, 0u, 0u};
+            p.segs[s] = SegDesc{-1, 0, 0u, 0u};
       }
 
       Slice<R> xs, acc;
@@ -817,7 +828,9 @@ __global__ __launch_bounds__(kBlockThreads) void rows_kernel(const Params<IdxT> 
          for (int r = 0; r < R; r++) acc.v[r] = zero4();
       }
 
-      walk_edges<V, L, R, EXACT, OP, SOPK, U, IdxT>(acc, xs, p, jb, je, lane, tab);
+      EdgeChunk<IdxT> chunk;
+      load_chunk<OP, IdxT>(chunk, p, jb, je, lane);
+      walk_edges<V, L, R, EXACT, OP, SOPK, U, IdxT>(acc, xs, p, jb, je, chunk, (IdxT)0, (IdxT)0, lane, tab);
       merge_subwaves<L, R, OP>(acc, p.imessage);
 
       if (sub == 0)
@@ -853,18 +866,34 @@ __global__ __launch_bounds__(kBlockThreads) void segments_kernel(const Params<Id
    const bool reads_x = op_reads_x<OP>(p.imessage);
    const int aop = p.imessage & 0xF0000;
 
+   // Segments are dealt round-robin to the waves, so the next one is known: its
+   // descriptor is fetched while the current segment is walked, and its first 64
+   // column ids while the current segment's last chunk is gathered.
+   auto fetch_desc = [&](int64_t q) -> SegDesc {
+      if (q < (int64_t)nseg) return p.segs[q];
+      return SegDesc{-1, 0, 0u, 0u};
+   };
+   SegDesc sd = fetch_desc(wave0);
+   EdgeChunk<IdxT> chunk;
+   {
+      const IdxT b0 = (IdxT)wave_uniform<int64_t>(sd.first);
+      const IdxT n0 = (IdxT)__builtin_amdgcn_readfirstlane((int)sd.count);
+      load_chunk<OP, IdxT>(chunk, p, b0, b0 + n0, lane);
+   }
    for (int64_t q = wave0; q < (int64_t)nseg; q += nwaves)
    {
-      const SegDesc sd = p.segs[q];
       const int64_t row = wave_uniform<int64_t>(sd.row);
-      const unsigned int seg = (unsigned int)__builtin_amdgcn_readfirstlane((int)sd.seg);
-      if (row < 0) continue;   // slot of a row that was handled inline
-      const IdxT rb = wave_uniform<IdxT>(p.pntrb[row]);
-      const IdxT re = wave_uniform<IdxT>(p.pntre[row]);
-      const IdxT seg_len = (IdxT)__builtin_amdgcn_readfirstlane((int)sd.len);
-      const IdxT jb = rb + (IdxT)seg * seg_len;
-      IdxT je = jb + seg_len;
-      if (je > re) je = re;
+      const IdxT jb = (IdxT)wave_uniform<int64_t>(sd.first);
+      const IdxT je = jb + (IdxT)__builtin_amdgcn_readfirstlane((int)sd.count);
+      const SegDesc sdn = fetch_desc(q + nwaves);
+      if (row < 0)
+      {
+         // slot of a row that was handled inline: nothing to do but keep the pipeline fed
+         const IdxT nb = (IdxT)wave_uniform<int64_t>(sdn.first);
+         load_chunk<OP, IdxT>(chunk, p, nb, nb + (IdxT)__builtin_amdgcn_readfirstlane((int)sdn.count), lane);
+         sd = sdn;
+         continue;
+      }
 
       Slice<R> xs, acc;
       if (reads_x) load_slice<V, L, R, EXACT, true>(xs, p.x + row * p.ldx, sl, p.k);
@@ -877,10 +906,16 @@ __global__ __launch_bounds__(kBlockThreads) void segments_kernel(const Params<Id
 #pragma unroll
       for (int r = 0; r < R; r++) acc.v[r] = real4{id, id, id, id};
 
-      walk_edges<V, L, R, EXACT, OP, SOPK, U, IdxT>(acc, xs, p, jb, je, lane, tab);
+      // the descriptor of the next segment was requested before this walk's first
+      // gather, so it has arrived by the time the walk asks for the next chunk
+      // (kept per-lane, not made wave-uniform here: that would wait for it now)
+      const IdxT nb = (IdxT)sdn.first;
+      const IdxT ne = nb + (IdxT)sdn.count;
+      walk_edges<V, L, R, EXACT, OP, SOPK, U, IdxT>(acc, xs, p, jb, je, chunk, nb, ne, lane, tab);
       merge_subwaves<L, R, OP>(acc, p.imessage);
 
       if (sub == 0) store_slice<V, L, R, EXACT>(p.partial + (int64_t)q * p.kpad, acc, sl, p.k);
+      sd = sdn;
    }
 }
 
