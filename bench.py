@@ -35,6 +35,7 @@ WORKLOADS = {
     "c3": ("spmm K=256, R-MAT scale 22 edge factor 16, symmetrised", "m", 256, None),
     "c3g": ("gcn K=256, R-MAT scale 22 edge factor 16, symmetrised", "g", 256, None),
     "c4": ("tdist K=64, R-MAT scale 24 edge factor 16, symmetrised", "t", 64, "tdist"),
+    "c4g": ("gcn K=64 on the c4 graph (same gathers, no reduction or scalar op)", "g", 64, None),
     "c5": ("sigmoid K=512, Zipf(1.8) degrees n=2^21 nnz~4e7, hubs to 1e6", "s", 512, "sigmoid"),
 }
 
@@ -57,7 +58,7 @@ def make_workload(name, scale_down=0):
         g = synth.rmat_graph(22 - sd, 16, 3)
         g["val"] = synth.edge_values(g["nnz"], 3)
         return g, None, synth.normal_matrix(g["rows"], 256, 3)
-    if name == "c4":
+    if name in ("c4", "c4g"):
         g = synth.rmat_graph(24 - sd, 16, 4)
         n = g["rows"]
         return g, synth.uniform_matrix(n, 64, -1.0, 1.0, 4, 1), synth.uniform_matrix(n, 64, -1.0, 1.0, 4, 2)

@@ -802,6 +802,20 @@ __global__ __launch_bounds__(kBlockThreads) void rows_kernel(const Params<IdxT> 
             p.segs[s] = SegDesc{-1, 0, 0u, 0u};
       }
 
+      real_t *zrow = p.z + row * p.ldz;
+      if (deg <= 0)
+      {
+         // empty row (about half the rows of an R-MAT graph): nothing to gather; the
+         // overwrite rule still clears Z, every other rule leaves it alone
+         if (!generic && p.beta_zero && sub == 0)
+         {
+            Slice<R> zero;
+#pragma unroll
+            for (int r = 0; r < R; r++) zero.v[r] = zero4();
+            store_slice<V, L, R, EXACT, true>(zrow, zero, sl, p.k);
+         }
+         continue;
+      }
       Slice<R> xs, acc;
       if (reads_x) load_slice<V, L, R, EXACT, true>(xs, p.x + row * p.ldx, sl, p.k);
       else
@@ -809,7 +823,6 @@ __global__ __launch_bounds__(kBlockThreads) void rows_kernel(const Params<IdxT> 
 #pragma unroll
          for (int r = 0; r < R; r++) xs.v[r] = zero4();
       }
-      real_t *zrow = p.z + row * p.ldz;
       if (generic)
       {
          // general semantics: fold the edges into the caller's Z with AOP
