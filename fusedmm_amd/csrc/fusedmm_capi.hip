@@ -249,7 +249,9 @@ int launch_instance(const Params<idx_t> &p, const Launch &l)
    int64_t gr = (int64_t)l.num_cu * (l.blocks_per_cu > 0 ? l.blocks_per_cu : occ_rows);
    if (gr > need) gr = need;
    Params<idx_t> pr = p;
-   pr.row_counters = (gr * kWavesPerBlock >= kRowCounters) ? kRowCounters : 1;
+   const int64_t nchunks = (p.m + kRowsPerClaim - 1) / kRowsPerClaim;
+   if (nchunks <= gr * kWavesPerBlock) pr.row_counters = 0;   // one chunk per wave at most: static
+   else pr.row_counters = (gr * kWavesPerBlock >= kRowCounters) ? kRowCounters : 1;
    const int64_t gs = (int64_t)l.num_cu * (l.blocks_per_cu > 0 ? l.blocks_per_cu : occ_segs);
    if (l.ev) FMM_HIP(hipEventRecord(l.ev[0], l.stream));
    hipLaunchKernelGGL((rows_kernel<V, L, R, EXACT, OP, SOPK, U, idx_t>), dim3((unsigned int)gr), dim3(kBlockThreads), 0, l.stream, pr);

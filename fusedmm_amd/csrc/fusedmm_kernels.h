@@ -103,7 +103,7 @@ struct Params {
    real_t *partial;        // [cap_seg][kpad]
    unsigned int cap_heavy, cap_seg;
    int kpad;
-   int row_counters;       // claim counters in use: kRowCounters, or 1 when the grid has fewer waves
+   int row_counters;       // claim counters in use: kRowCounters; 1 when the grid has fewer waves; 0: wave w takes chunk w
 };
 
 // ---- wave primitives --------------------------------------------------------
@@ -741,12 +741,20 @@ __global__ __launch_bounds__(kBlockThreads) void rows_kernel(const Params<IdxT> 
    // then looks at all counters with one vector load and moves to the next one
    // that still has chunks.  The next claim is issued before the current rows
    // are walked, so its latency is hidden.
-   const int nc = p.row_counters;                        // 64, or 1 for tiny grids
+   // Small inputs (no more chunks than waves in the grid): row_counters == 0 and
+   // wave w simply takes chunk w -- nothing to balance, no counter traffic.
+   const int nc = p.row_counters;                        // 64, 1 for tiny grids, 0: static
    const int64_t nchunks = (p.m + kRowsPerClaim - 1) / kRowsPerClaim;
-   int cur = (int)((blockIdx.x * kWavesPerBlock + (threadIdx.x >> 6)) & (unsigned)(nc - 1));
+   const int64_t wave_id = (int64_t)blockIdx.x * kWavesPerBlock + (threadIdx.x >> 6);
+   int cur = nc > 0 ? (int)(wave_id & (unsigned)(nc - 1)) : 0;
    unsigned long long claimed = 0;
-   if (lane == 0) claimed = atomicAdd(&p.ctr->rows[cur].next, 1ull);
-   int64_t chunk = resolve_claim<IdxT>(p, claimed, cur, nc, nchunks, lane);
+   int64_t chunk;
+   if (nc == 0) chunk = wave_id < nchunks ? wave_id : -1;
+   else
+   {
+      if (lane == 0) claimed = atomicAdd(&p.ctr->rows[cur].next, 1ull);
+      chunk = resolve_claim<IdxT>(p, claimed, cur, nc, nchunks, lane);
+   }
    while (chunk >= 0)
    {
    const int64_t row0 = chunk * kRowsPerClaim;
@@ -756,7 +764,7 @@ __global__ __launch_bounds__(kBlockThreads) void rows_kernel(const Params<IdxT> 
       my_b = p.pntrb[row0 + lane];
       my_e = p.pntre[row0 + lane];
    }
-   if (lane == 0) claimed = atomicAdd(&p.ctr->rows[cur].next, 1ull);
+   if (nc > 0 && lane == 0) claimed = atomicAdd(&p.ctr->rows[cur].next, 1ull);
    for (int t = 0; t < kRowsPerClaim && row0 + t < p.m; t++)
    {
       const int64_t row = row0 + t;
@@ -857,7 +865,7 @@ __global__ __launch_bounds__(kBlockThreads) void rows_kernel(const Params<IdxT> 
          store_slice<V, L, R, EXACT, true>(zrow, acc, sl, p.k);
       }
    }
-   chunk = resolve_claim<IdxT>(p, claimed, cur, nc, nchunks, lane);
+   chunk = nc > 0 ? resolve_claim<IdxT>(p, claimed, cur, nc, nchunks, lane) : -1;
    }
 }
 
