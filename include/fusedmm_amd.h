@@ -49,7 +49,10 @@ void fusedMM_amd_set_sop_callback(fusedMM_amd_sop_fn fn);
  * work is enqueued on `stream` (a hipStream_t; NULL is the default stream) and
  * the call returns without waiting.  No counterpart in the reference; it is what
  * a framework that already keeps its tensors on the GPU binds (the reference's
- * CMakeLists.txt:1-14 packages fusedMM_csr for DGL).  FUSEDMM_SOP_KIND_HOST is
+ * CMakeLists.txt:1-14 packages fusedMM_csr for DGL).  Every call on a GPU uses
+ * that GPU's one set of work queues: calls enqueued on different streams must
+ * not overlap in time (use one stream, or order them with events).
+ * FUSEDMM_SOP_KIND_HOST is
  * not available here (it needs the host between passes): returns
  * FUSEDMM_UNDEFINED_USER_FUNCTION.
  */
