@@ -1,0 +1,38 @@
+"""bench.py host-side contract that needs no GPU."""
+import os
+import subprocess
+import sys
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def test_more_than_one_gpu_is_refused_with_a_message():
+    r = subprocess.run([sys.executable, os.path.join(ROOT, "bench.py"), "--gpus", "2"],
+                       stdout=subprocess.PIPE, stderr=subprocess.PIPE, text=True, timeout=60)
+    assert r.returncode == 2 and "ONE GPU" in r.stderr and r.stdout == ""
+
+
+def test_algorithmic_bytes_formula_matches_the_stated_c2_figure():
+    sys.path.insert(0, ROOT)
+    from fusedmm_amd import synth
+    # nnz (4K + I) + m (4K [X] + 4K [Z] + 2I):  2^24 * 516 + 2^20 * 1032
+    assert synth.algorithmic_bytes("s", 1 << 20, 128, 1 << 24, 4) == 9739173888
+    assert synth.algorithmic_bytes("m", 10, 256, 100, 4) == 100 * (1024 + 4 + 4) + 10 * (1024 + 8)
+    assert synth.algorithmic_flops("s", 128, 1 << 24) == 4 * 128 * (1 << 24)
+
+
+def test_scaled_workloads_have_the_advertised_shape():
+    sys.path.insert(0, ROOT)
+    import bench
+    g, X, Y = bench.make_workload("c2", 8)
+    assert g["rows"] == 4096 and g["nnz"] == 65536 and X.shape == (4096, 128) and X is not Y
+    deg = np.diff(g["rowptr"])
+    rid = np.repeat(np.arange(4096), deg)
+    assert (g["indx"] != rid).all()                                   # no self loops
+    assert all(np.all(np.diff(g["indx"][a:b]) > 0) for a, b in zip(g["rowptr"][:50], g["rowptr"][1:51]))  # sorted, distinct
+    g, X, Y = bench.make_workload("c1", 4)
+    assert X is Y and np.abs(X).max() <= 1.0                          # A = B, U[-1, 1]
+    g, _, _ = bench.make_workload("c5", 6)
+    assert np.diff(g["rowptr"]).max() == min(1000000, (1 << 15) // 2)  # hubs at the cap
