@@ -1,0 +1,86 @@
+"""Seeded random sweep over shapes, strides, index widths, precisions, tuples and
+split thresholds, each checked against the CPU oracle."""
+import numpy as np
+import pytest
+
+import checks
+import fusedmm_amd as fa
+import gpu_api
+import graphs
+from oracle_api import MSG, SOP_NAMES, Oracle
+
+pytestmark = pytest.mark.gpu
+_ORC = {}
+
+
+def orc(vbits):
+    if vbits not in _ORC:
+        _ORC[vbits] = Oracle(vbits=vbits)
+    return _ORC[vbits]
+
+
+@pytest.mark.parametrize("seed", range(48))
+def test_random_pattern_case(seed):
+    rng = np.random.default_rng(1000 + seed)
+    bits = int(rng.choice([32, 64]))
+    vbits = int(rng.choice([32, 64]))
+    np_v = np.float32 if vbits == 32 else np.float64
+    rows, cols = int(rng.integers(1, 90)), int(rng.integers(1, 120))
+    k = int(rng.choice([1, 2, 3, 4, 5, 8, 12, 31, 32, 33, 64, 100, 128, 200, 256, 300, 512, 640]))
+    hub = int(rng.choice([0, 5, 70, 900]))
+    tkern, kind = [("g", None), ("m", None), ("s", "sigmoid"), ("t", "tdist"), ("f", "fr"), ("s", "ll"), ("t", "fa")][seed % 7]
+    beta = float(rng.choice([0.0, 1.0]))
+    # a ragged graph with arbitrary (possibly repeated, unsorted) columns
+    lists = [rng.integers(0, cols, int(rng.integers(0, 9))) for _ in range(rows)]
+    if hub and rows > 2:
+        lists[int(rng.integers(0, rows))] = rng.integers(0, cols, hub)
+    deg = np.array([len(x) for x in lists], np.int64)
+    rowptr = np.concatenate([[0], np.cumsum(deg)])
+    from fusedmm_amd import synth
+    g = synth.graph_from_rowptr(rows, cols, rowptr, np.concatenate(lists) if deg.sum() else np.zeros(0, np.int64), None, bits)
+    g["val"] = synth.edge_values(max(1, g["nnz"]), seed)[:g["nnz"]] if g["nnz"] else np.zeros(1, np.float32)
+    if g["nnz"] == 0:
+        g["indx"] = np.zeros(1, g["indx"].dtype)
+    if rng.random() < 0.4 and g["nnz"] > 0:
+        g = graphs.split_pointers(g, seed)
+    pad = lambda: int(rng.choice([0, 0, 1, 3, 4]))
+    ldx, ldy, ldz = k + pad(), k + pad(), k + pad()
+    lo, hi = (0.1, 1.0) if kind in ("fr", "fa", "ll") else (-0.5, 0.5) if tkern == "s" else (-1.0, 1.0)
+    X = graphs.features(rows, ldx, seed, lo, hi, 1).astype(np_v)
+    # distance tuples with 1/s or sqrt bodies: keep X and Y apart (s > 0); the dot tuple with log2(1+sqrt): s > 0
+    far = kind in ("fr", "fa", "ll") and tkern != "s"
+    Y = graphs.features(cols, ldy, seed, -hi if far else lo, -lo if far else hi, 2).astype(np_v)
+    Z0 = graphs.features(rows, ldz, seed, -1, 1, 3).astype(np_v)
+    m = rows if rng.random() < 0.7 else int(rng.integers(0, rows + 1))
+    sk = SOP_NAMES[kind] if kind else 0
+    where = "device" if rng.random() < 0.7 else "host"
+    split = None if rng.random() < 0.5 else (int(rng.integers(1, 40)), int(rng.integers(1, 20)))
+    print("case", seed, dict(bits=bits, vbits=vbits, rows=rows, cols=cols, k=k, hub=hub, op=tkern, kind=kind, beta=beta,
+                             ld=(ldx, ldy, ldz), m=m, where=where, split=split), flush=True)
+    gpu_api.set_kind(sk, bits, vbits)
+    if split:
+        gpu_api.set_split(split[0], split[1], bits, vbits)
+    try:
+        rc, Z = gpu_api.run(MSG[tkern], g, X, Y, Z0, beta=beta, bits=bits, where=where, m=m, k=k, ldx=ldx, ldy=ldy,
+                            ldz=ldz, vbits=vbits)
+    finally:
+        gpu_api.set_split(0, 0, bits, vbits)
+    assert rc == 0
+    o = orc(vbits)
+    want = Z0.copy()
+    assert 0 == o.opt("t" if tkern == "f" else tkern, g, X, Y, want, beta=beta, sop_kind=sk, mode=1, m=m, k=k, ldx=ldx, ldy=ldy, ldz=ldz)
+    # rows >= m and padding columns untouched
+    np.testing.assert_array_equal(Z[m:], Z0[m:])
+    np.testing.assert_array_equal(Z[:, k:], Z0[:, k:])
+    eps = float(np.finfo(np_v).eps)
+    scale = float(np.abs(want[:m, :k]).max()) + 1.0 if m else 1.0
+    tol = 64 * eps * max(1, hub, 9) * scale
+    extra = None
+    if kind == "sigmoid":
+        gg = dict(g)
+        extra_full, _ = checks.sigmoid_flip_slack(o.table().astype(np.float32), gg, X[:, :k].astype(np.float64), Y[:, :k].astype(np.float64), m)
+        extra = np.zeros((rows, k))
+        extra[:m] = extra_full
+    err = np.abs(Z[:, :k].astype(np.float64) - want[:, :k].astype(np.float64))
+    bound = tol + (extra if extra is not None else 0.0)
+    assert np.all(err <= bound), (float(err.max()), tol)
