@@ -84,3 +84,43 @@ def test_random_pattern_case(seed):
     err = np.abs(Z[:, :k].astype(np.float64) - want[:, :k].astype(np.float64))
     bound = tol + (extra if extra is not None else 0.0)
     assert np.all(err <= bound), (float(err.max()), tol)
+
+
+@pytest.mark.parametrize("seed", range(32))
+def test_random_general_tuple(seed):
+    """Any non-UDEF stage combination (plus SOP_UDEF with a device body), through
+    the run-time switched kernel, against the oracle's restatement of the
+    reference's general pipeline."""
+    rng = np.random.default_rng(5000 + seed)
+    bits = int(rng.choice([32, 64]))
+    vbits = int(rng.choice([32, 64]))
+    np_v = np.float32 if vbits == 32 else np.float64
+    k = int(rng.choice([3, 8, 20, 64, 96, 130, 256]))
+    g = graphs.ragged(bits, seed=seed + 1, rows=int(rng.integers(5, 60)), cols=int(rng.integers(30, 90)),
+                      hub_deg=int(rng.choice([10, 200])), hub_rows=(3,))
+    vop = int(rng.integers(1, 8))
+    rop = int(rng.choice([0x00, 0x10, 0x20, 0x30, 0x40, 0x50]))
+    sop, vsc = [(0x100, 0x1000), (0x100, 0x2000), (0xF00, 0x1000), (0x000, 0x0000), (0xF00, 0x2000)][int(rng.integers(0, 5))]
+    aop = int(rng.choice([0x10000, 0x20000, 0x30000, 0x00000]))
+    imsg = vop | rop | sop | vsc | aop
+    X = graphs.features(g["rows"], k, seed, -1, 1, 1).astype(np_v)
+    Y = graphs.features(g["cols"], k, seed, -1, 1, 2).astype(np_v)
+    Z0 = graphs.features(g["rows"], k, seed, -1, 1, 3).astype(np_v)
+    split = None if rng.random() < 0.5 else (6, 5)
+    print("case", seed, hex(imsg), dict(bits=bits, vbits=vbits, k=k, split=split), flush=True)
+    lib = fa.load(bits, vbits)
+    gpu_api.set_kind(SOP_NAMES["tdist"], bits, vbits)
+    prev = lib.fusedMM_amd_set_opt(0)
+    if split:
+        gpu_api.set_split(split[0], split[1], bits, vbits)
+    try:
+        rc, Z = gpu_api.run(imsg, g, X, Y, Z0, bits=bits, vbits=vbits)
+    finally:
+        lib.fusedMM_amd_set_opt(prev)
+        gpu_api.set_split(0, 0, bits, vbits)
+    assert rc == 0
+    want = Z0.copy()
+    assert orc(vbits).generic(imsg, g, X, Y, want, sop_kind=SOP_NAMES["tdist"]) == 0
+    eps = float(np.finfo(np_v).eps)
+    tol = 256 * eps * 200 * (float(np.abs(want).max()) + 1.0)
+    assert float(np.abs(Z.astype(np.float64) - want.astype(np.float64)).max()) <= tol
