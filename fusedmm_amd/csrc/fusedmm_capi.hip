@@ -70,7 +70,7 @@ struct DeviceState {
    int num_cu = 0;
    val_t *sigmoid_table = nullptr;
    Counters *ctr = nullptr;
-   Buffer heavy, segs, partial;
+   Buffer heavy, segs, partial, queued;
    Buffer stage[8];           // host-pointer mode: pntrb, pntre, indx, val, x, y, z, spare
    // timing
    hipEvent_t ev[kTimingSlots][4];
@@ -229,6 +229,7 @@ int pick_shape(int k, bool vec_ok, Shape *s)
 
 struct Launch {
    int num_cu, blocks_per_cu;
+   int64_t nnz_hint;
    hipStream_t stream;
    hipEvent_t *ev;   // 4 events or nullptr
 };
@@ -236,27 +237,31 @@ struct Launch {
 template <int V, int L, int R, bool EXACT, int OP, int SOPK, int U>
 int launch_instance(const Params<idx_t> &p, const Launch &l)
 {
-   // persistent grids: as many blocks as stay resident, each wave strides over rows
-   static int occ_rows = 0, occ_segs = 0;
-   if (occ_rows == 0)
+   // persistent grid: as many blocks as stay resident; waves share out the
+   // queued segments, then claim rows
+   static int occ = 0;
+   if (occ == 0)
    {
-      FMM_HIP(hipOccupancyMaxActiveBlocksPerMultiprocessor(&occ_rows, rows_kernel<V, L, R, EXACT, OP, SOPK, U, idx_t>, kBlockThreads, 0));
-      FMM_HIP(hipOccupancyMaxActiveBlocksPerMultiprocessor(&occ_segs, segments_kernel<V, L, R, EXACT, OP, SOPK, U, idx_t>, kBlockThreads, 0));
-      if (occ_rows < 1) occ_rows = 1;
-      if (occ_segs < 1) occ_segs = 1;
+      FMM_HIP(hipOccupancyMaxActiveBlocksPerMultiprocessor(&occ, fused_kernel<V, L, R, EXACT, OP, SOPK, U, idx_t>, kBlockThreads, 0));
+      if (occ < 1) occ = 1;
    }
-   const int64_t need = (p.m + kWavesPerBlock - 1) / kWavesPerBlock;
-   int64_t gr = (int64_t)l.num_cu * (l.blocks_per_cu > 0 ? l.blocks_per_cu : occ_rows);
+   // enough blocks for the rows, or for the segments the caller's nnz could give rise to
+   int64_t need = (p.m + kWavesPerBlock - 1) / kWavesPerBlock;
+   const int64_t need_segs = (l.nnz_hint / p.seg_len + kWavesPerBlock - 1) / kWavesPerBlock;
+   if (need < need_segs) need = need_segs;
+   int64_t gr = (int64_t)l.num_cu * (l.blocks_per_cu > 0 ? l.blocks_per_cu : occ);
    if (gr > need) gr = need;
+   if (gr < 1) gr = 1;
    Params<idx_t> pr = p;
    const int64_t nchunks = (p.m + kRowsPerClaim - 1) / kRowsPerClaim;
    if (nchunks <= gr * kWavesPerBlock) pr.row_counters = 0;   // one chunk per wave at most: static
    else pr.row_counters = (gr * kWavesPerBlock >= kRowCounters) ? kRowCounters : 1;
-   const int64_t gs = (int64_t)l.num_cu * (l.blocks_per_cu > 0 ? l.blocks_per_cu : occ_segs);
+   int64_t gc = (p.m + kBlockThreads - 1) / kBlockThreads;
+   if (gc > (int64_t)l.num_cu * 8) gc = (int64_t)l.num_cu * 8;
    if (l.ev) FMM_HIP(hipEventRecord(l.ev[0], l.stream));
-   hipLaunchKernelGGL((rows_kernel<V, L, R, EXACT, OP, SOPK, U, idx_t>), dim3((unsigned int)gr), dim3(kBlockThreads), 0, l.stream, pr);
+   hipLaunchKernelGGL((classify_kernel<idx_t>), dim3((unsigned int)gc), dim3(kBlockThreads), 0, l.stream, p);
    if (l.ev) FMM_HIP(hipEventRecord(l.ev[1], l.stream));
-   hipLaunchKernelGGL((segments_kernel<V, L, R, EXACT, OP, SOPK, U, idx_t>), dim3((unsigned int)gs), dim3(kBlockThreads), 0, l.stream, p);
+   hipLaunchKernelGGL((fused_kernel<V, L, R, EXACT, OP, SOPK, U, idx_t>), dim3((unsigned int)gr), dim3(kBlockThreads), 0, l.stream, pr);
    if (l.ev) FMM_HIP(hipEventRecord(l.ev[2], l.stream));
    hipLaunchKernelGGL((merge_kernel<idx_t>), dim3((unsigned int)(l.num_cu * 2)), dim3(kBlockThreads), 0, l.stream, p, (int)(OP == OP_GENERIC));
    if (l.ev) FMM_HIP(hipEventRecord(l.ev[3], l.stream));
@@ -378,10 +383,12 @@ int run_slab(const Args &a, const Plan &pl, int sop_kind, hipStream_t stream)
    p.imessage = a.imessage;
    p.sigmoid_table = d->sigmoid_table;
 
-   // heavy-row split: segments of about 1 MiB of gathered rows (measured best on the
-   // R-MAT and power-law benchmark graphs: shorter segments pay their start-up and
-   // partial-result cost more often, longer ones leave long rows to single waves)
+   // heavy-row split: segments of about 1 MiB of gathered rows but at most 2048 edges
+   // (measured best on the R-MAT and power-law benchmark graphs: shorter segments pay
+   // their start-up and partial-result cost more often, longer ones leave long rows
+   // to single waves)
    int seg_len = g.seg_len > 0 ? g.seg_len : (int)(1048576 / ((int64_t)kValBytes * a.k));
+   if (g.seg_len <= 0 && seg_len > 2048) seg_len = 2048;
    if (seg_len < 64 && g.seg_len <= 0) seg_len = 64;
    int64_t heavy_deg = g.heavy_deg > 0 ? g.heavy_deg : 2 * (int64_t)seg_len;
    if (heavy_deg < seg_len) heavy_deg = seg_len;
@@ -402,18 +409,27 @@ int run_slab(const Args &a, const Plan &pl, int sop_kind, hipStream_t stream)
    st = grow(d->heavy, (size_t)cap_heavy * sizeof(HeavyRow)); if (st) return st;
    st = grow(d->segs, (size_t)cap_seg * sizeof(SegDesc)); if (st) return st;
    st = grow(d->partial, (size_t)cap_seg * p.kpad * kValBytes); if (st) return st;
+   const int64_t queued_words = (a.m + 31) / 32;
+   st = grow(d->queued, (size_t)queued_words * sizeof(unsigned int)); if (st) return st;
    p.ctr = d->ctr;
    p.heavy = (HeavyRow *)d->heavy.ptr;
    p.segs = (SegDesc *)d->segs.ptr;
    p.partial = (val_t *)d->partial.ptr;
+   p.queued = (unsigned int *)d->queued.ptr;
    p.cap_heavy = (unsigned int)cap_heavy;
    p.cap_seg = (unsigned int)cap_seg;
 
-   hipLaunchKernelGGL(reset_counters_kernel, dim3(1), dim3(kBlockThreads), 0, stream, d->ctr);
+   {
+      int64_t rb = (queued_words + kBlockThreads - 1) / kBlockThreads;
+      if (rb > (int64_t)d->num_cu * 4) rb = (int64_t)d->num_cu * 4;
+      if (rb < 1) rb = 1;
+      hipLaunchKernelGGL(reset_kernel, dim3((unsigned int)rb), dim3(kBlockThreads), 0, stream, d->ctr, p.queued, queued_words);
+   }
 
    Launch l;
    l.num_cu = d->num_cu;
    l.blocks_per_cu = g.blocks_per_cu;
+   l.nnz_hint = nnz_hint;
    l.stream = stream;
    l.ev = nullptr;
    if (g.timing && g.timing_calls < kTimingSlots)
@@ -959,7 +975,7 @@ void fusedMM_amd_timing(int enable)
    g.timing_calls = 0;
 }
 
-int fusedMM_amd_timing_summary(double *rows_ms, double *segments_ms, double *merge_ms)
+int fusedMM_amd_timing_summary(double *classify_ms, double *fused_ms, double *merge_ms)
 {
    std::lock_guard<std::mutex> lock(g.mu);
    double t[3] = {0, 0, 0};
@@ -976,8 +992,8 @@ int fusedMM_amd_timing_summary(double *rows_ms, double *segments_ms, double *mer
             t[e] += ms;
          }
    }
-   if (rows_ms) *rows_ms = t[0];
-   if (segments_ms) *segments_ms = t[1];
+   if (classify_ms) *classify_ms = t[0];
+   if (fused_ms) *fused_ms = t[1];
    if (merge_ms) *merge_ms = t[2];
    return n;
 }
@@ -1022,7 +1038,7 @@ void fusedMM_amd_finalize(void)
       (void)hipDeviceSynchronize();
       (void)hipFree(d.sigmoid_table);
       (void)hipFree(d.ctr);
-      Buffer *bufs[] = {&d.heavy, &d.segs, &d.partial};
+      Buffer *bufs[] = {&d.heavy, &d.segs, &d.partial, &d.queued};
       for (Buffer *b : bufs) { if (b->ptr) (void)hipFree(b->ptr); *b = Buffer(); }
       for (Buffer &b : d.stage) { if (b.ptr) (void)hipFree(b.ptr); b = Buffer(); }
       if (d.ev_made)

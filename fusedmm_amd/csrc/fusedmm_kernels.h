@@ -101,6 +101,7 @@ struct Params {
    HeavyRow *heavy;
    SegDesc *segs;
    real_t *partial;        // [cap_seg][kpad]
+   unsigned int *queued;   // one bit per row: set by the classify kernel for rows it put on the heavy-row queue
    unsigned int cap_heavy, cap_seg;
    int kpad;
    int row_counters;       // claim counters in use: kRowCounters; 1 when the grid has fewer waves; 0: wave w takes chunk w
@@ -718,167 +719,55 @@ __device__ __forceinline__ int64_t resolve_claim(const Params<IdxT> &p, unsigned
    }
 }
 
-// ---- kernel 1: one wavefront per row, heavy rows queued -------------------------
-template <int V, int L, int R, bool EXACT, int OP, int SOPK, int U, typename IdxT>
-__global__ __launch_bounds__(kBlockThreads) void rows_kernel(const Params<IdxT> p)
+// ---- kernel 1: put heavy rows on the queue -----------------------------------------
+// One thread per row; reads the row pointers only.  A row with more than
+// heavy_deg edges gets a HeavyRow entry and one SegDesc per segment (at most
+// kMaxSegsPerRow: hub rows get longer segments) and its bit in `queued` is set.
+// When the queue is full the row is left for phase B to process whole.
+template <typename IdxT>
+__global__ __launch_bounds__(kBlockThreads) void classify_kernel(const Params<IdxT> p)
 {
-   constexpr int S = 64 / L;
-   __shared__ real_t lds_tab[(OP >= OP_DOT) ? kSigmoidTableSize : 1];
-   const bool uses_sop = (OP == OP_DOT || OP == OP_DIST || (OP == OP_GENERIC && (p.imessage & 0xF00) == kSopUdef));
-   const real_t *tab = stage_table(p.sigmoid_table, lds_tab, (OP >= OP_DOT) && uses_sop && (SOPK >= 0 ? SOPK : p.sop_kind) == SOP_SIGMOID);
-
-   const int lane = threadIdx.x & 63;
-   const int sub = lane / L, sl = lane % L;
-   const bool reads_x = op_reads_x<OP>(p.imessage);
-   const int aop = p.imessage & 0xF0000;
-   const bool generic = (OP == OP_GENERIC);
-
-   // Rows are claimed dynamically in chunks of kRowsPerClaim: degree-skewed
-   // graphs (R-MAT, power law) leave any static row -> wave map unbalanced.
-   // Counter c hands out, in round t, chunk  t * nc + ((c ^ mix(t)) & (nc-1)):
-   // every chunk has one owner, and a counter's chunks do not share row-id
-   // bits (R-MAT degrees depend on them).  A wave drains its home counter,
-   // then looks at all counters with one vector load and moves to the next one
-   // that still has chunks.  The next claim is issued before the current rows
-   // are walked, so its latency is hidden.
-   // Small inputs (no more chunks than waves in the grid): row_counters == 0 and
-   // wave w simply takes chunk w -- nothing to balance, no counter traffic.
-   const int nc = p.row_counters;                        // 64, 1 for tiny grids, 0: static
-   const int64_t nchunks = (p.m + kRowsPerClaim - 1) / kRowsPerClaim;
-   const int64_t wave_id = (int64_t)blockIdx.x * kWavesPerBlock + (threadIdx.x >> 6);
-   int cur = nc > 0 ? (int)(wave_id & (unsigned)(nc - 1)) : 0;
-   unsigned long long claimed = 0;
-   int64_t chunk;
-   if (nc == 0) chunk = wave_id < nchunks ? wave_id : -1;
-   else
+   const int64_t stride = (int64_t)gridDim.x * kBlockThreads;
+   for (int64_t row = (int64_t)blockIdx.x * kBlockThreads + threadIdx.x; row < p.m; row += stride)
    {
-      if (lane == 0) claimed = atomicAdd(&p.ctr->rows[cur].next, 1ull);
-      chunk = resolve_claim<IdxT>(p, claimed, cur, nc, nchunks, lane);
-   }
-   while (chunk >= 0)
-   {
-   const int64_t row0 = chunk * kRowsPerClaim;
-   IdxT my_b = 0, my_e = 0;   // lane t holds the pointers of row0 + t
-   if (lane < kRowsPerClaim && row0 + lane < p.m)
-   {
-      my_b = p.pntrb[row0 + lane];
-      my_e = p.pntre[row0 + lane];
-   }
-   if (nc > 0 && lane == 0) claimed = atomicAdd(&p.ctr->rows[cur].next, 1ull);
-   for (int t = 0; t < kRowsPerClaim && row0 + t < p.m; t++)
-   {
-      const int64_t row = row0 + t;
-      const IdxT jb = lane_value<IdxT>(my_b, t);
-      const IdxT je = lane_value<IdxT>(my_e, t);
-      const int64_t deg = (int64_t)je - (int64_t)jb;
-
-      if (deg > p.heavy_deg)
+      const IdxT jb = p.pntrb[row];
+      const int64_t deg = (int64_t)p.pntre[row] - (int64_t)jb;
+      if (deg <= p.heavy_deg) continue;
+      int64_t seg_len = p.seg_len;
+      if (deg > seg_len * (int64_t)kMaxSegsPerRow) seg_len = (deg + kMaxSegsPerRow - 1) / kMaxSegsPerRow;
+      const unsigned int nseg = (unsigned int)((deg + seg_len - 1) / seg_len);
+      const unsigned int slot = atomicAdd(&p.ctr->n_heavy, 1u);
+      const unsigned int base = atomicAdd(&p.ctr->n_seg, nseg);
+      if (slot < p.cap_heavy && (uint64_t)base + nseg <= (uint64_t)p.cap_seg)
       {
-         // queue the row for the segment kernel; if the queue is full, fall through
-         // at most kMaxSegsPerRow partials per row: hub rows get longer segments
-         int64_t seg_len = p.seg_len;
-         if (deg > seg_len * (int64_t)kMaxSegsPerRow) seg_len = (deg + kMaxSegsPerRow - 1) / kMaxSegsPerRow;
-         unsigned int nseg = (unsigned int)((deg + seg_len - 1) / seg_len);
-         unsigned int slot = 0, base = 0;
-         if (lane == 0)
+         p.heavy[slot] = HeavyRow{row, base, nseg};
+         for (unsigned int s = 0; s < nseg; s++)
          {
-            slot = atomicAdd(&p.ctr->n_heavy, 1u);
-            base = atomicAdd(&p.ctr->n_seg, nseg);
+            const int64_t off = (int64_t)s * seg_len;
+            const int64_t cnt = deg - off < seg_len ? deg - off : seg_len;
+            p.segs[base + s] = SegDesc{row, (int64_t)jb + off, (unsigned int)cnt, 0u};
          }
-         slot = (unsigned int)__builtin_amdgcn_readfirstlane((int)slot);
-         base = (unsigned int)__builtin_amdgcn_readfirstlane((int)base);
-         const bool fits = slot < p.cap_heavy && (uint64_t)base + nseg <= (uint64_t)p.cap_seg;
-         if (fits)
-         {
-            if (lane == 0) p.heavy[slot] = HeavyRow{row, base, nseg};
-            for (unsigned int s = lane; s < nseg; s += 64)
-            {
-               const int64_t off = (int64_t)s * seg_len;
-               const int64_t cnt = deg - off < seg_len ? deg - off : seg_len;
-               p.segs[base + s] = SegDesc{row, (int64_t)jb + off, (unsigned int)cnt, 0u};
-            }
-            continue;
-         }
-         // mark the slot unused (the merge kernel skips n_seg == 0) and do the row here
-         if (lane == 0)
-         {
-            if (slot < p.cap_heavy) p.heavy[slot] = HeavyRow{row, 0u, 0u};
-            atomicAdd(&p.ctr->overflow, 1u);
-         }
-         // every queue entry below the cap has exactly one writer: poison ours
-         for (uint64_t s = (uint64_t)base + lane; s < (uint64_t)base + nseg && s < (uint64_t)p.cap_seg; s += 64)
+         atomicOr(&p.queued[row >> 5], 1u << (row & 31));
+      }
+      else
+      {
+         // slot unused (the merge kernel skips n_seg == 0); every queue entry below the
+         // cap has exactly one writer: poison ours
+         if (slot < p.cap_heavy) p.heavy[slot] = HeavyRow{row, 0u, 0u};
+         atomicAdd(&p.ctr->overflow, 1u);
+         for (uint64_t s = base; s < (uint64_t)base + nseg && s < (uint64_t)p.cap_seg; s++)
             p.segs[s] = SegDesc{-1, 0, 0u, 0u};
       }
-
-      real_t *zrow = p.z + row * p.ldz;
-      if (deg <= 0)
-      {
-         // empty row (about half the rows of an R-MAT graph): nothing to gather; the
-         // overwrite rule still clears Z, every other rule leaves it alone
-         if (!generic && p.beta_zero && sub == 0)
-         {
-            Slice<R> zero;
-#pragma unroll
-            for (int r = 0; r < R; r++) zero.v[r] = zero4();
-            store_slice<V, L, R, EXACT, true>(zrow, zero, sl, p.k);
-         }
-         continue;
-      }
-      Slice<R> xs, acc;
-      if (reads_x) load_slice<V, L, R, EXACT, true>(xs, p.x + row * p.ldx, sl, p.k);
-      else
-      {
-#pragma unroll
-         for (int r = 0; r < R; r++) xs.v[r] = zero4();
-      }
-      if (generic)
-      {
-         // general semantics: fold the edges into the caller's Z with AOP
-         if (aop == kAopNoop) continue;
-         if (sub == 0) load_slice<V, L, R, EXACT>(acc, zrow, sl, p.k);
-         else
-         {
-            const real_t id = aop_identity(aop);
-#pragma unroll
-            for (int r = 0; r < R; r++) acc.v[r] = real4{id, id, id, id};
-         }
-      }
-      else
-      {
-#pragma unroll
-         for (int r = 0; r < R; r++) acc.v[r] = zero4();
-      }
-
-      EdgeChunk<IdxT> chunk;
-      load_chunk<OP, IdxT>(chunk, p, jb, je, lane);
-      walk_edges<V, L, R, EXACT, OP, SOPK, U, IdxT>(acc, xs, p, jb, je, chunk, (IdxT)0, (IdxT)0, lane, tab);
-      merge_subwaves<L, R, OP>(acc, p.imessage);
-
-      if (sub == 0)
-      {
-         if (!generic && !p.beta_zero)
-         {
-            Slice<R> zin;
-            load_slice<V, L, R, EXACT>(zin, zrow, sl, p.k);
-            map2(acc, zin, acc, [](real_t a, real_t b) { return a + b; });
-         }
-         store_slice<V, L, R, EXACT, true>(zrow, acc, sl, p.k);
-      }
-   }
-   chunk = nc > 0 ? resolve_claim<IdxT>(p, claimed, cur, nc, nchunks, lane) : -1;
    }
 }
 
-// ---- kernel 2: one wavefront per queued edge segment -> partial Z -----------------
+// ---- phase A of the fused kernel: one wavefront per queued edge segment -> partial Z ----
 template <int V, int L, int R, bool EXACT, int OP, int SOPK, int U, typename IdxT>
-__global__ __launch_bounds__(kBlockThreads) void segments_kernel(const Params<IdxT> p)
+__device__ __forceinline__ void segments_phase(const Params<IdxT> &p, const real_t *tab)
 {
-   __shared__ real_t lds_tab[(OP >= OP_DOT) ? kSigmoidTableSize : 1];
    unsigned int nseg = p.ctr->n_seg;
-   if (nseg > p.cap_seg) nseg = p.cap_seg;   // rows beyond the cap were done inline
+   if (nseg > p.cap_seg) nseg = p.cap_seg;   // rows beyond the cap are done whole in phase B
    if (nseg == 0) return;
-   const bool uses_sop = (OP == OP_DOT || OP == OP_DIST || (OP == OP_GENERIC && (p.imessage & 0xF00) == kSopUdef));
-   const real_t *tab = stage_table(p.sigmoid_table, lds_tab, (OP >= OP_DOT) && uses_sop && (SOPK >= 0 ? SOPK : p.sop_kind) == SOP_SIGMOID);
 
    const int lane = threadIdx.x & 63;
    const int sub = lane / L, sl = lane % L;
@@ -938,6 +827,137 @@ __global__ __launch_bounds__(kBlockThreads) void segments_kernel(const Params<Id
       if (sub == 0) store_slice<V, L, R, EXACT>(p.partial + (int64_t)q * p.kpad, acc, sl, p.k);
       sd = sdn;
    }
+}
+
+// ---- phase B of the fused kernel: one wavefront per row ---------------------------
+template <int V, int L, int R, bool EXACT, int OP, int SOPK, int U, typename IdxT>
+__device__ __forceinline__ void rows_phase(const Params<IdxT> &p, const real_t *tab)
+{
+   const int lane = threadIdx.x & 63;
+   const int sub = lane / L, sl = lane % L;
+   const bool reads_x = op_reads_x<OP>(p.imessage);
+   const int aop = p.imessage & 0xF0000;
+   const bool generic = (OP == OP_GENERIC);
+
+   // Rows are claimed dynamically in chunks of kRowsPerClaim: degree-skewed
+   // graphs (R-MAT, power law) leave any static row -> wave map unbalanced.
+   // Counter c hands out, in round t, chunk  t * nc + ((c ^ mix(t)) & (nc-1)):
+   // every chunk has one owner, and a counter's chunks do not share row-id
+   // bits (R-MAT degrees depend on them).  A wave drains its home counter,
+   // then looks at all counters with one vector load and moves to the next one
+   // that still has chunks.  The next claim is issued before the current rows
+   // are walked, so its latency is hidden.
+   // Small inputs (no more chunks than waves in the grid): row_counters == 0 and
+   // wave w simply takes chunk w -- nothing to balance, no counter traffic.
+   const int nc = p.row_counters;                        // 64, 1 for tiny grids, 0: static
+   const int64_t nchunks = (p.m + kRowsPerClaim - 1) / kRowsPerClaim;
+   const int64_t wave_id = (int64_t)blockIdx.x * kWavesPerBlock + (threadIdx.x >> 6);
+   int cur = nc > 0 ? (int)(wave_id & (unsigned)(nc - 1)) : 0;
+   unsigned long long claimed = 0;
+   int64_t chunk;
+   if (nc == 0) chunk = wave_id < nchunks ? wave_id : -1;
+   else
+   {
+      if (lane == 0) claimed = atomicAdd(&p.ctr->rows[cur].next, 1ull);
+      chunk = resolve_claim<IdxT>(p, claimed, cur, nc, nchunks, lane);
+   }
+   while (chunk >= 0)
+   {
+   const int64_t row0 = chunk * kRowsPerClaim;
+   IdxT my_b = 0, my_e = 0;   // lane t holds the pointers of row0 + t
+   if (lane < kRowsPerClaim && row0 + lane < p.m)
+   {
+      my_b = p.pntrb[row0 + lane];
+      my_e = p.pntre[row0 + lane];
+   }
+   if (nc > 0 && lane == 0) claimed = atomicAdd(&p.ctr->rows[cur].next, 1ull);
+   for (int t = 0; t < kRowsPerClaim && row0 + t < p.m; t++)
+   {
+      const int64_t row = row0 + t;
+      const IdxT jb = lane_value<IdxT>(my_b, t);
+      const IdxT je = lane_value<IdxT>(my_e, t);
+      const int64_t deg = (int64_t)je - (int64_t)jb;
+
+      if (deg > p.heavy_deg)
+      {
+         // queued by the classify kernel and already walked, segment by segment, in
+         // phase A -- unless the queue was full, in which case the row is done here
+         const unsigned int word = p.queued[row >> 5];
+         if ((word >> (row & 31)) & 1u) continue;
+      }
+
+      real_t *zrow = p.z + row * p.ldz;
+      if (deg <= 0)
+      {
+         // empty row (about half the rows of an R-MAT graph): nothing to gather; the
+         // overwrite rule still clears Z, every other rule leaves it alone
+         if (!generic && p.beta_zero && sub == 0)
+         {
+            Slice<R> zero;
+#pragma unroll
+            for (int r = 0; r < R; r++) zero.v[r] = zero4();
+            store_slice<V, L, R, EXACT, true>(zrow, zero, sl, p.k);
+         }
+         continue;
+      }
+      Slice<R> xs, acc;
+      if (reads_x) load_slice<V, L, R, EXACT, true>(xs, p.x + row * p.ldx, sl, p.k);
+      else
+      {
+#pragma unroll
+         for (int r = 0; r < R; r++) xs.v[r] = zero4();
+      }
+      if (generic)
+      {
+         // general semantics: fold the edges into the caller's Z with AOP
+         if (aop == kAopNoop) continue;
+         if (sub == 0) load_slice<V, L, R, EXACT>(acc, zrow, sl, p.k);
+         else
+         {
+            const real_t id = aop_identity(aop);
+#pragma unroll
+            for (int r = 0; r < R; r++) acc.v[r] = real4{id, id, id, id};
+         }
+      }
+      else
+      {
+#pragma unroll
+         for (int r = 0; r < R; r++) acc.v[r] = zero4();
+      }
+
+      EdgeChunk<IdxT> first;
+      load_chunk<OP, IdxT>(first, p, jb, je, lane);
+      walk_edges<V, L, R, EXACT, OP, SOPK, U, IdxT>(acc, xs, p, jb, je, first, (IdxT)0, (IdxT)0, lane, tab);
+      merge_subwaves<L, R, OP>(acc, p.imessage);
+
+      if (sub == 0)
+      {
+         if (!generic && !p.beta_zero)
+         {
+            Slice<R> zin;
+            load_slice<V, L, R, EXACT>(zin, zrow, sl, p.k);
+            map2(acc, zin, acc, [](real_t a, real_t b) { return a + b; });
+         }
+         store_slice<V, L, R, EXACT, true>(zrow, acc, sl, p.k);
+      }
+   }
+   chunk = nc > 0 ? resolve_claim<IdxT>(p, claimed, cur, nc, nchunks, lane) : -1;
+   }
+}
+
+// ---- kernel 2: the fused SDDMM+SpMM kernel ------------------------------------------
+// Long work first: every wave takes its share of the queued segments of heavy
+// rows (phase A), then claims ordinary rows until none are left (phase B).  One
+// kernel, so the short rows fill in behind the long segments instead of waiting
+// for them at a kernel boundary.
+template <int V, int L, int R, bool EXACT, int OP, int SOPK, int U, typename IdxT>
+__global__ __launch_bounds__(kBlockThreads) void fused_kernel(const Params<IdxT> p)
+{
+   __shared__ real_t lds_tab[(OP >= OP_DOT) ? kSigmoidTableSize : 1];
+   const bool uses_sop = (OP == OP_DOT || OP == OP_DIST || (OP == OP_GENERIC && (p.imessage & 0xF00) == kSopUdef));
+   const real_t *tab = stage_table(p.sigmoid_table, lds_tab, (OP >= OP_DOT) && uses_sop && (SOPK >= 0 ? SOPK : p.sop_kind) == SOP_SIGMOID);
+   segments_phase<V, L, R, EXACT, OP, SOPK, U, IdxT>(p, tab);
+   rows_phase<V, L, R, EXACT, OP, SOPK, U, IdxT>(p, tab);
 }
 
 // ---- kernel 3: fold the partials of each heavy row -------------------------------------
@@ -1087,12 +1107,18 @@ __global__ __launch_bounds__(kBlockThreads) void zero_rows_kernel(real_t *z, int
       z[(i / k) * ldz + (i % k)] = (real_t)0;
 }
 
-// Clears the queue and claim counters before each call.  A kernel rather than a
-// memset so that callers may capture the stream entry point in a HIP graph.
-__global__ __launch_bounds__(kBlockThreads) void reset_counters_kernel(Counters *c)
+// Clears the queue and claim counters and the queued-row bitmap before each call.
+// A kernel rather than a memset so that callers may capture the stream entry
+// point in a HIP graph.
+__global__ __launch_bounds__(kBlockThreads) void reset_kernel(Counters *c, unsigned int *queued, int64_t words)
 {
-   unsigned int *w = reinterpret_cast<unsigned int *>(c);
-   for (unsigned int i = threadIdx.x; i < sizeof(Counters) / sizeof(unsigned int); i += kBlockThreads) w[i] = 0u;
+   if (blockIdx.x == 0)
+   {
+      unsigned int *w = reinterpret_cast<unsigned int *>(c);
+      for (unsigned int i = threadIdx.x; i < sizeof(Counters) / sizeof(unsigned int); i += kBlockThreads) w[i] = 0u;
+   }
+   for (int64_t i = (int64_t)blockIdx.x * kBlockThreads + threadIdx.x; i < words; i += (int64_t)gridDim.x * kBlockThreads)
+      queued[i] = 0u;
 }
 
 // Plain 16-byte copy of known size: the yardstick the HBM traffic counters

@@ -119,10 +119,11 @@ void fusedMM_amd_set_split(int64_t heavy_deg, int seg_len);
  * Per-kernel timing with HIP events on the stream the kernels run on.
  * enable != 0 starts a fresh recording (up to 512 calls are kept); the summary
  * waits for the recorded events and returns the number of calls and the summed
- * milliseconds of the row kernel, the segment kernel and the merge kernel.
+ * milliseconds of the three kernels of a call: classify (queues heavy rows),
+ * fused (all the gathering and arithmetic), merge (folds split rows).
  */
 void fusedMM_amd_timing(int enable);
-int fusedMM_amd_timing_summary(double *rows_ms, double *segments_ms, double *merge_ms);
+int fusedMM_amd_timing_summary(double *classify_ms, double *fused_ms, double *merge_ms);
 
 /* Counters of the last call on this thread's device: heavy rows queued, edge
  * segments queued, heavy rows that did not fit the queue.  Waits for the device. */

@@ -29,7 +29,7 @@ MAX_SEGS_PER_ROW = 512   # kMaxSegsPerRow of the kernels: longer rows get longer
 
 def default_split(k, vbits=32):
     """(heavy_deg, seg_len) defaults of the library for feature width k."""
-    seg = max(64, 1048576 // ((vbits // 8) * k))
+    seg = max(64, min(2048, 1048576 // ((vbits // 8) * k)))
     return 2 * seg, seg
 
 
