@@ -397,7 +397,7 @@ int run_slab(const Args &a, const Plan &pl, int sop_kind, hipStream_t stream)
    p.kpad = (int)((a.k + 3) / 4 * 4);
 
    // queue capacities from the caller's nnz when it is plausible; rows that do
-   // not fit are processed whole by the row kernel, so this is never a
+   // not fit are processed whole in the row phase, so this is never a
    // correctness question
    int64_t nnz_hint = (a.nnz > 0 && a.nnz < ((int64_t)1 << 40)) ? a.nnz : (int64_t)1 << 26;
    int64_t cap_seg = nnz_hint / seg_len * 3 / 2 + 1024;   // a row of d edges has at most d/seg_len + 1 segments

@@ -2,8 +2,8 @@
 //
 // One wavefront walks one CSR row (or one fixed-length edge segment of a heavy
 // row).  A wavefront is cut into S = 64/L sub-waves of L lanes; a sub-wave owns
-// one neighbour row Y[c] at a time, each lane holding R float4 slices of it, so
-// a gather is L coalesced 16-byte loads.  The X[i] slice and the Z accumulator
+// one neighbour row Y[c] at a time, each lane holding R four-element slices of
+// it, so a gather is L coalesced 16-byte loads (two per lane in double precision).  The X[i] slice and the Z accumulator
 // live in VGPRs for the whole row.  The per-edge reduction (ROP) is a DPP /
 // swizzle XOR butterfly over the L lanes, the scalar op (SOP) and the scaled
 // accumulate (MOP, AOP) happen in registers.
@@ -52,9 +52,9 @@ constexpr int kBlockThreads = 256;
 constexpr int kWavesPerBlock = kBlockThreads / 64;
 
 struct Counters {
-   unsigned int n_heavy;    // heavy rows queued by the row kernel
+   unsigned int n_heavy;    // heavy rows queued by the classify kernel
    unsigned int n_seg;      // edge segments queued
-   unsigned int overflow;   // heavy rows that did not fit the queue (handled inline)
+   unsigned int overflow;   // heavy rows that did not fit the queue (processed whole in phase B)
    unsigned int invalid;    // set by the optional operand check
    unsigned int pad2[28];         // keep the row counters on their own 128-byte lines
    // Row claim counters.  Read-modify-writes on ONE address retire one per

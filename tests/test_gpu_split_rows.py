@@ -82,7 +82,7 @@ def test_default_thresholds_hub_row(oracle, tkern, kind):
 
 def test_queue_overflow_is_handled_inline(oracle):
     """A caller-supplied nnz that is far too small undersizes the segment queue:
-    rows that do not fit are processed whole by the row kernel; the answer stays right."""
+    rows that do not fit are processed whole in the row phase; the answer stays right."""
     bits, k = 32, 64
     g = graphs.ragged(bits, rows=40, cols=3000, hub_deg=2000, hub_rows=(11, 13, 17))
     Y = graphs.features(g["cols"], k, 3, -0.5, 0.5, 2)
