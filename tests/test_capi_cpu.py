@@ -74,3 +74,18 @@ def test_sop_kind_selection():
     assert lib.fusedMM_amd_get_sop_kind() == fa.SOP_KIND_FR
     lib.fusedMM_amd_set_sop_kind(prev)
     assert lib.fusedMM_amd_set_opt(1) in (0, 1)
+
+
+@pytest.mark.parametrize("idx,val", [("int32_t", "float"), ("int64_t", "float"), ("int64_t", "double")])
+@pytest.mark.parametrize("compiler,std", [("gcc", "-std=c99"), ("g++", "-std=c++11")])
+def test_headers_compile_as_plain_c_and_cpp(tmp_path, compiler, std, idx, val):
+    """The boundary is a C ABI: both headers must compile as C99 and as C++11 with
+    nothing but INDEXTYPE / VALUETYPE defined, as the reference's header does."""
+    import subprocess
+    src = tmp_path / ("t.c" if compiler == "gcc" else "t.cpp")
+    src.write_text('#include <stdint.h>\n#include "fusedMM.h"\n#include "fusedmm_amd.h"\n'
+                   'int probe(void) { return VOP_COPY_RHS | ROP_DOT | SOP_UDEF | VSC_MUL | AOP_ADD; }\n')
+    r = subprocess.run([compiler, std, "-Wall", "-Wextra", "-Werror", "-pedantic", "-fsyntax-only",
+                        "-DINDEXTYPE=" + idx, "-DVALUETYPE=" + val, "-I", os.path.join(ROOT, "include"), str(src)],
+                       stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
+    assert r.returncode == 0, r.stdout
