@@ -173,6 +173,11 @@ def main():
     wall = time.perf_counter() - t0
     r_ms, s_ms, g_ms = C.c_double(), C.c_double(), C.c_double()
     ncalls = lib.fusedMM_amd_timing_summary(C.byref(r_ms), C.byref(s_ms), C.byref(g_ms))
+    per_call = []
+    for i in range(max(0, ncalls)):
+        c_, f_, m_ = C.c_double(), C.c_double(), C.c_double()
+        if lib.fusedMM_amd_timing_call(i, C.byref(c_), C.byref(f_), C.byref(m_)) == 0:
+            per_call.append(c_.value + f_.value + m_.value)
     lib.fusedMM_amd_timing(0)
     ms_per_step = wall / args.steps * 1e3
 
@@ -232,6 +237,8 @@ def main():
         "hbm_GBps_algorithmic": b_alg / (ms_per_step * 1e-3) / 1e9,
         "pct_peak_hbm": 100.0 * b_alg / (ms_per_step * 1e-3) / 1e9 / PEAK_HBM_GBPS,
         "kernel_ms": kern_ms,
+        "kernels_ms_per_call": {"min": float(np.min(per_call)), "median": float(np.median(per_call)),
+                                "max": float(np.max(per_call))} if per_call else None,
         "split": {"heavy_rows": hs[0].value, "segments": hs[1].value, "overflow": hs[2].value},
         "spot_check_vs_oracle": checked,
         "roofline": roofline,

@@ -35,7 +35,7 @@ NOT_ENOUGH_MEM, UNDEFINED_USER_FUNCTION, NO_OPT_IMPL = -1, 64, 128
 EXPORTS = ("fusedMM_csr", "fusedMM_csr_stream", "fusedMM_amd_index_bytes", "fusedMM_amd_value_bytes",
            "fusedMM_amd_set_sop_kind", "fusedMM_amd_get_sop_kind", "fusedMM_amd_set_sop_callback",
            "fusedMM_amd_set_opt", "fusedMM_amd_set_validate", "fusedMM_amd_set_split", "fusedMM_amd_timing",
-           "fusedMM_amd_timing_summary", "fusedMM_amd_last_split", "fusedMM_amd_copy_probe",
+           "fusedMM_amd_timing_summary", "fusedMM_amd_timing_call", "fusedMM_amd_last_split", "fusedMM_amd_copy_probe",
            "fusedMM_amd_finalize")
 
 _libs = {}
@@ -83,6 +83,8 @@ def load(index_bits=32, value_bits=32):
     lib.fusedMM_amd_timing.argtypes = [C.c_int]
     lib.fusedMM_amd_timing_summary.argtypes = [C.POINTER(C.c_double)] * 3
     lib.fusedMM_amd_timing_summary.restype = C.c_int
+    lib.fusedMM_amd_timing_call.argtypes = [C.c_int] + [C.POINTER(C.c_double)] * 3
+    lib.fusedMM_amd_timing_call.restype = C.c_int
     lib.fusedMM_amd_last_split.argtypes = [C.POINTER(C.c_uint)] * 3
     lib.fusedMM_amd_last_split.restype = C.c_int
     lib.fusedMM_amd_copy_probe.argtypes = [vp, vp, C.c_int64, vp]

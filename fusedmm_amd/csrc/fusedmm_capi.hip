@@ -998,6 +998,22 @@ int fusedMM_amd_timing_summary(double *classify_ms, double *fused_ms, double *me
    return n;
 }
 
+int fusedMM_amd_timing_call(int i, double *classify_ms, double *fused_ms, double *merge_ms)
+{
+   std::lock_guard<std::mutex> lock(g.mu);
+   if (i < 0 || i >= g.timing_calls) return FUSEDMM_FAIL_RETURN;
+   DeviceState &d = g.dev[g.timing_dev];
+   if (hipEventSynchronize(d.ev[i][3]) != hipSuccess) return FUSEDMM_FAIL_RETURN;
+   double *out[3] = {classify_ms, fused_ms, merge_ms};
+   for (int e = 0; e < 3; e++)
+   {
+      float ms = 0.f;
+      if (hipEventElapsedTime(&ms, d.ev[i][e], d.ev[i][e + 1]) != hipSuccess) return FUSEDMM_FAIL_RETURN;
+      if (out[e]) *out[e] = ms;
+   }
+   return FUSEDMM_SUCCESS_RETURN;
+}
+
 int fusedMM_amd_last_split(unsigned int *heavy_rows, unsigned int *segments, unsigned int *overflow)
 {
    std::lock_guard<std::mutex> lock(g.mu);

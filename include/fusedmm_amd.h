@@ -124,6 +124,8 @@ void fusedMM_amd_set_split(int64_t heavy_deg, int seg_len);
  */
 void fusedMM_amd_timing(int enable);
 int fusedMM_amd_timing_summary(double *classify_ms, double *fused_ms, double *merge_ms);
+/* The same for recorded call number i (0-based); returns 0, or FUSEDMM_FAIL_RETURN when i is out of range. */
+int fusedMM_amd_timing_call(int i, double *classify_ms, double *fused_ms, double *merge_ms);
 
 /* Counters of the last call on this thread's device: heavy rows queued, edge
  * segments queued, heavy rows that did not fit the queue.  Waits for the device. */
