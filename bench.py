@@ -114,7 +114,7 @@ def main():
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py: this path is built and measured on ONE GPU; --gpus %d is not supported "
-              "(rows are independent, see DESIGN.md for how it would shard)" % args.gpus, file=sys.stderr)
+              "(rows are independent: a sharded run would split the rows of A, X and Z across GPUs)" % args.gpus, file=sys.stderr)
         sys.exit(2)
 
     import torch
