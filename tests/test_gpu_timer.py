@@ -73,3 +73,21 @@ def test_sweep_script(tmp_path):
     lines = open(str(tmp_path / "res" / "tiny-s-sreal-gpu.csv")).read().strip().splitlines()
     assert lines[0].startswith("Filename,NNZ") and len(lines) == 9
     assert [l.split(",")[4] for l in lines[1:]] == ["32", "64", "96", "128", "160", "192", "224", "256"]
+
+
+def test_config1_through_the_timer(tmp_path):
+    """Benchmark configuration 1 end to end, the way the reference runs it
+    (x..time_fr -input file.mtx -T 1 -K 32): symmetric ER graph with 16 384 nodes
+    and 131 072 undirected pairs written as .mtx from seed, loaded by the timer's
+    own loader, FR op, tester on, then timed."""
+    from bench import make_workload
+    g, _, _ = make_workload("c1")
+    path = str(tmp_path / "c1.mtx")
+    synth.write_mtx_symmetric(path, g)
+    exe = os.path.join(str(tmp_path), "xsOptFusedMMtime_fr_pt")     # the reference's executable name selects the kind
+    os.symlink(fbuild.timer_path(64), exe)
+    r = subprocess.run([exe, "-input", path, "-T", "1", "-K", "32", "-nrep", "5"],
+                       stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True, timeout=200)
+    assert r.returncode == 0 and "PASSED TEST" in r.stdout, r.stdout
+    f = r.stdout.strip().splitlines()[-1].split(",")
+    assert f[1:5] == ["262144", "16384", "16384", "32"]
