@@ -249,7 +249,11 @@ int launch_instance(const Params<idx_t> &p, const Launch &l)
    int64_t need = (p.m + kWavesPerBlock - 1) / kWavesPerBlock;
    const int64_t need_segs = (l.nnz_hint / p.seg_len + kWavesPerBlock - 1) / kWavesPerBlock;
    if (need < need_segs) need = need_segs;
-   int64_t gr = (int64_t)l.num_cu * (l.blocks_per_cu > 0 ? l.blocks_per_cu : occ);
+   // Four workgroups (16 waves) per CU at most: with 8-16 gathers in flight per wave
+   // that saturates the memory system, and more waves only evict each other's lines
+   // (measured on the sigmoid K=128 benchmark: 1.307 ms at 4 per CU, 1.314 at 5, 1.335 at 6).
+   const int resident = occ < 4 ? occ : 4;
+   int64_t gr = (int64_t)l.num_cu * (l.blocks_per_cu > 0 ? l.blocks_per_cu : resident);
    if (gr > need) gr = need;
    if (gr < 1) gr = 1;
    Params<idx_t> pr = p;
