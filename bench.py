@@ -26,7 +26,7 @@ PEAK_HBM_GBPS = 8000.0
 # WRITE_SIZE, each scaled by the same counter's reading for a plain 1 GiB copy
 # (one summary per workload under profiles/).  Measured, not computed: refreshed
 # whenever the kernel changes.
-MEASURED_TRAFFIC_BYTES = {"c2": 9808124314, "c3": 125575561662, "c4": 129192668055, "c5": 90428018444}
+MEASURED_TRAFFIC_BYTES = {"c2": 9759204040, "c3": 125575561662, "c4": 129057569729, "c5": 90428018444}
 
 WORKLOADS = {
     # name: (description, op letter, K, sop kind)
