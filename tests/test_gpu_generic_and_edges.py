@@ -269,3 +269,21 @@ def test_mixed_host_and_device_operands_are_refused():
     assert rc == fa.FAIL
     torch.cuda.synchronize()
     assert not Zd.any()
+
+
+def test_finalize_releases_and_the_library_recovers(oracle):
+    """fusedMM_amd_finalize() frees every buffer the library holds; the next call
+    sets everything up again (table, counters, queues)."""
+    g = graphs.ragged(32, hub_deg=5000)
+    k = 64
+    X = graphs.features(g["rows"], k, 3, -0.5, 0.5, 1)
+    Y = graphs.features(g["cols"], k, 3, -0.5, 0.5, 2)
+    Z0 = np.zeros((g["rows"], k), np.float32)
+    gpu_api.set_kind(SOP_NAMES["sigmoid"], 32)
+    rc, Za = gpu_api.run(MSG["s"], g, X, Y, Z0)
+    assert rc == 0
+    fa.load(32).fusedMM_amd_finalize()
+    fa.load(32).fusedMM_amd_finalize()          # twice is harmless
+    rc, Zb = gpu_api.run(MSG["s"], g, X, Y, Z0, where="host")
+    assert rc == 0
+    np.testing.assert_array_equal(Za.view(np.uint32), Zb.view(np.uint32))
