@@ -1,5 +1,7 @@
 """Seeded random sweep over shapes, strides, index widths, precisions, tuples and
 split thresholds, each checked against the CPU oracle."""
+import os
+
 import numpy as np
 import pytest
 
@@ -11,6 +13,8 @@ from oracle_api import MSG, SOP_NAMES, Oracle
 
 pytestmark = pytest.mark.gpu
 _ORC = {}
+# FUSEDMM_TEST_SEEDS=<n> widens both sweeps (default: 48 pattern cases, 32 general tuples)
+_N = int(os.environ.get("FUSEDMM_TEST_SEEDS", "0"))
 
 
 def orc(vbits):
@@ -19,7 +23,7 @@ def orc(vbits):
     return _ORC[vbits]
 
 
-@pytest.mark.parametrize("seed", range(48))
+@pytest.mark.parametrize("seed", range(_N or 48))
 def test_random_pattern_case(seed):
     rng = np.random.default_rng(1000 + seed)
     bits = int(rng.choice([32, 64]))
@@ -86,7 +90,7 @@ def test_random_pattern_case(seed):
     assert np.all(err <= bound), (float(err.max()), tol)
 
 
-@pytest.mark.parametrize("seed", range(32))
+@pytest.mark.parametrize("seed", range(_N or 32))
 def test_random_general_tuple(seed):
     """Any non-UDEF stage combination (plus SOP_UDEF with a device body), through
     the run-time switched kernel, against the oracle's restatement of the
