@@ -3,8 +3,8 @@
 // One wavefront walks one CSR row (or one fixed-length edge segment of a heavy
 // row).  A wavefront is cut into S = 64/L sub-waves of L lanes; a sub-wave owns
 // one neighbour row Y[c] at a time, each lane holding R four-element slices of
-// it, so a gather is L coalesced 16-byte loads (two per lane in double precision).  The X[i] slice and the Z accumulator
-// live in VGPRs for the whole row.  The per-edge reduction (ROP) is a DPP /
+// it, so a gather is L coalesced 16-byte loads (two per lane in double
+// precision).  The X[i] slice and the Z accumulator live in VGPRs for the whole row.  The per-edge reduction (ROP) is a DPP /
 // swizzle XOR butterfly over the L lanes, the scalar op (SOP) and the scaled
 // accumulate (MOP, AOP) happen in registers.
 //
