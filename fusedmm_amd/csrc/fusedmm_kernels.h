@@ -556,13 +556,12 @@ struct EdgeChunk {
 template <int OP, typename IdxT>
 __device__ __forceinline__ void load_chunk(EdgeChunk<IdxT> &c, const Params<IdxT> &p, IdxT j0, IdxT je, int lane)
 {
-   const IdxT j = j0 + lane;
    c.col = 0;
    c.val = (real_t)0;
-   if (j < je)
+   if (j0 < je && (IdxT)lane < je - j0)   // written so that an int32 slot number next to 2^31 cannot wrap
    {
-      c.col = p.indx[j];
-      if ((OP == OP_SPMM || OP == OP_GENERIC) && p.val) c.val = p.val[j];
+      c.col = p.indx[j0 + lane];
+      if ((OP == OP_SPMM || OP == OP_GENERIC) && p.val) c.val = p.val[j0 + lane];
    }
 }
 
@@ -614,12 +613,13 @@ __device__ __forceinline__ void walk_edges(Slice<R> &acc, const Slice<R> &xs, co
       load_chunk<OP, IdxT>(cur, p, next_b, next_e, lane);
       return;
    }
-   for (IdxT j0 = jb; j0 < je; j0 += 64)
+   for (IdxT j0 = jb; j0 < je;)
    {
       EdgeChunk<IdxT> nxt;
-      if (j0 + 64 < je) load_chunk<OP, IdxT>(nxt, p, j0 + 64, je, lane);
+      const IdxT left = je - j0;          // > 0; comparisons on differences: no wrap next to 2^31
+      if (left > 64) load_chunk<OP, IdxT>(nxt, p, j0 + 64, je, lane);
       else load_chunk<OP, IdxT>(nxt, p, next_b, next_e, lane);
-      const int n = (je - j0) < 64 ? (int)(je - j0) : 64;
+      const int n = left < 64 ? (int)left : 64;
       for (int b0 = 0; b0 < n; b0 += S * U)
       {
          IdxT col[U];
@@ -642,6 +642,8 @@ __device__ __forceinline__ void walk_edges(Slice<R> &acc, const Slice<R> &xs, co
             if (ok[u]) edge_step<L, R, OP>(acc, xs, ys[u], ev[u], sop_kind, p.imessage, tab);
       }
       cur = nxt;
+      if (left <= 64) break;
+      j0 += 64;
    }
 }
 
