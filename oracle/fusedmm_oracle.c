@@ -22,10 +22,16 @@
  *          inputs; scipy CSR @ Y for the spmm/gcn tuples; dense brute force.
  *   orc_fusedmm_opt_*      - golden Z from the reference harness's trusted
  *          kernels and generic fusedMM_csr; dense fp64 brute force; invariants.
- *   orc_partition_rows_*   - hand-computed examples and properties (ranges tile
- *          [0,m) in order, bounded imbalance).  The reference does not expose its
- *          partition, so no vector of its own pins this one: PARITY UNPINNED
- *          beyond those checks.  Only the CPU baseline's thread ranges use it.
+ *   orc_partition_rows_*   - row for row against the thread the real reference
+ *          (fusedMM.c built with -DPTTIME -DLOAD_BALANCE -DNTHREADS=2,3,5,8,16
+ *          plus ref_partition_probe.c, whose SOP_UDEF_FUNC records
+ *          omp_get_thread_num() per row) evaluates each row on: committed as
+ *          tests/golden/partition.npz (30 degree sets: front/back heavy, empty
+ *          rows at boundaries, fewer ranges than threads, m < rows, gapped
+ *          pointers, Zipf and geometric degrees) and live on fresh random sets
+ *          (tests/test_oracle_ref.py).  The vectors separate the rule from its
+ *          near misses (quota not recomputed, >= for >, tipping row kept, running
+ *          count not restarted); plus hand-computed examples.
  *   orc_gpu_dot / mode 2   - equals the fp64 dot within K*eps*sum|x*y|; equals
  *          the sequential dot exactly for inputs whose products are exactly
  *          representable (small integers), which a wrong lane map would break.

@@ -14,6 +14,11 @@ full so nothing has to be regenerated bit-for-bit) and the reference's outputs:
   tuples_i32.npz      Z of the reference's fusedMM_csr for a sweep of op tuples
   mtx.npz             CSR the reference's loader builds from hand-written .mtx
                       texts (stored alongside as strings)
+  partition.npz       which thread the reference's fusedMM_csr (built with its
+                      nnz-balanced row partition on 2, 3, 5, 8 and 16 threads)
+                      evaluated each row on, for the degree sets of
+                      graphs.partition_cases() (-1: a row without edges, whose
+                      holder the reference never shows)
 """
 import os
 import sys
@@ -26,7 +31,7 @@ sys.path.insert(0, os.path.dirname(HERE))
 sys.path.insert(0, os.path.dirname(os.path.dirname(HERE)))
 
 import graphs  # noqa: E402
-from oracle_api import MSG, Ref  # noqa: E402
+from oracle_api import MSG, PARTITION_THREADS, Ref, RefPartition  # noqa: E402
 
 KINDS = {"s": "sigmoid", "t": "tdist", "f": "fr", "m": "spmm", "g": "gcn"}
 
@@ -143,6 +148,18 @@ def main():
         out[name + "_shape"] = np.array([rows, cols])
         out[name + "_rowptr"], out[name + "_colids"], out[name + "_values"] = rowptr, colids, values
     np.savez_compressed(os.path.join(HERE, "mtx.npz"), **out)
+    out = {}
+    names = []
+    for name, pb, pe, m in graphs.partition_cases():
+        names.append(name)
+        out[name + "_pntrb"], out[name + "_pntre"], out[name + "_m"] = pb, pe, np.array(m)
+        for t in PARTITION_THREADS:
+            own32, _ = RefPartition(t, 32).owners(pb, pe, m)
+            own64, _ = RefPartition(t, 64).owners(pb, pe, m)
+            assert np.array_equal(own32, own64)
+            out["%s_owner_t%d" % (name, t)] = own32.astype(np.int8)
+    out["names"] = np.array(names)
+    np.savez_compressed(os.path.join(HERE, "partition.npz"), **out)
     print("golden fixtures written to", HERE)
 
 

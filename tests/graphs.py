@@ -74,3 +74,52 @@ def split_pointers(g, seed=5):
 
 def features(n, k, seed, lo=-0.5, hi=0.5, stream=1):
     return synth.uniform_matrix(n, k, lo, hi, seed, stream)
+
+
+def partition_cases():
+    """Row-degree sets for the nnz-balanced row partition (reference
+    fusedMM.c:633-676), as (name, pntrb, pntre, m) with int64 pointers.  Chosen so
+    that each step of the rule decides some case: the quota recomputed after
+    every closed range, the strict comparison, the tipping row opening the next
+    range, the running count restarting at zero, empty rows on either side of a
+    boundary, fewer ranges than threads, m < rows, pointers with gaps."""
+    cases = []
+
+    def add(name, deg, m=None):
+        deg = np.asarray(deg, np.int64)
+        ptr = np.concatenate([[0], np.cumsum(deg)]).astype(np.int64)
+        cases.append((name, ptr[:-1].copy(), ptr[1:].copy(), len(deg) if m is None else m))
+
+    add("front_heavy", [10] + [1] * 10)              # quota shrinks after the first range
+    add("back_heavy", [1] * 10 + [10])
+    add("hand", [3, 1, 1, 1, 3, 1])
+    add("hub_last_row", [0, 0, 0, 5])                # fewer ranges than threads
+    add("one_row", [7])
+    add("all_empty", [0] * 9)
+    add("ones16", [1] * 16)
+    add("ones17", [1] * 17)
+    add("exact_quota", [2, 2, 2, 2, 2, 2])           # running count EQUAL to the quota does not close a range
+    add("empties_at_boundaries", [4, 0, 0, 4, 0, 0, 4, 0, 0, 4, 0, 0, 4, 0])
+    add("empties_then_tip", [3, 0, 0, 0, 2, 0, 0, 3, 0, 1, 0, 0, 5, 0, 0, 1])
+    add("staircase", list(range(1, 40)))
+    add("staircase_down", list(range(39, 0, -1)))
+    add("m_less_than_rows", [5, 1, 1, 7, 2, 2, 9, 1, 1, 1, 30, 30], m=9)
+    rng = np.random.Generator(np.random.Philox(key=[77, 0]))
+    for n, cap in ((60, 50), (300, 80), (1000, 400), (2500, 2000)):
+        for rep in range(3):
+            deg = np.minimum(rng.zipf(1.5 + 0.2 * rep, n), cap)
+            deg[rng.random(n) < 0.3] = 0             # R-MAT graphs leave a third of the rows empty
+            add("zipf_n%d_%d" % (n, rep), deg)
+    for rep in range(3):
+        add("geometric_%d" % rep, rng.geometric(0.08, 500) - 1)
+    # rows stored with gaps and out of order: only pntre[i] - pntrb[i] may matter
+    deg = np.minimum(rng.zipf(1.7, 200), 60)
+    order = rng.permutation(200)
+    pb, pe = np.zeros(200, np.int64), np.zeros(200, np.int64)
+    pos = 3
+    for r in order:
+        pos += int(rng.integers(0, 4))
+        pb[r], pe[r] = pos, pos + int(deg[r])
+        pos = int(pe[r])
+    cases.append(("gapped_pointers", pb, pe, 200))
+    return cases

@@ -232,3 +232,62 @@ class Ref:
         values = np.empty(n.value, self.np_v)
         self.lib.ref_get_csr(_ptr(rowptr, self.ct), _ptr(colids, self.ct), _ptr(values, self.cv))
         return r.value, c.value, rowptr, colids, values
+
+
+PARTITION_THREADS = (2, 3, 5, 8, 16)   # PART_THREADS of oracle/Makefile
+
+
+def ref_partition_available(nthreads=8, bits=32):
+    return os.path.exists(os.path.join(ORACLE_DIR, "_ref", "libref_partition_t%d_i%d.so" % (nthreads, bits)))
+
+
+class RefPartition:
+    """The real reference's fusedMM.c built with its nnz-balanced row partition
+    (fusedMM.c:633-676) on `nthreads` threads, plus oracle/ref_partition_probe.c,
+    whose SOP_UDEF_FUNC records which thread evaluates each row."""
+
+    def __init__(self, nthreads, bits=32):
+        self.np_i, self.ct = _itype(bits)
+        self.nthreads = nthreads
+        self.lib = C.CDLL(os.path.join(ORACLE_DIR, "_ref", "libref_partition_t%d_i%d.so" % (nthreads, bits)))
+        assert self.lib.ref_probe_index_bytes() * 8 == bits and self.lib.ref_probe_threads() == nthreads
+
+    def owners(self, pntrb, pntre, m=None):
+        """(owner, calls): thread that evaluated each of the first m rows (-1 for
+        a row with no edge: the reference never shows who holds it) and the
+        number of edges it evaluated there."""
+        pntrb = np.ascontiguousarray(pntrb, self.np_i)
+        pntre = np.ascontiguousarray(pntre, self.np_i)
+        m = len(pntrb) if m is None else m
+        slots = int(pntre[:m].max()) if m else 0
+        val = np.zeros(max(slots, 1), np.float32)
+        for i in range(m):
+            val[int(pntrb[i]):int(pntre[i])] = i
+        indx = np.zeros(max(slots, 1), self.np_i)
+        x = np.zeros(max(m, 1), np.float32)
+        y = np.ones(1, np.float32)
+        z = np.zeros(max(m, 1), np.float32)
+        owner = np.full(max(m, 1), -1, np.int32)
+        calls = np.zeros(max(m, 1), np.int32)
+        fp, ip = C.POINTER(C.c_float), C.POINTER(self.ct)
+        fn = self.lib.ref_partition_probe
+        fn.restype = C.c_int
+        rc = fn(self.ct(m), self.ct(slots), _ptr(val, C.c_float), _ptr(indx, self.ct), _ptr(pntrb, self.ct),
+                _ptr(pntre, self.ct), _ptr(x, C.c_float), _ptr(y, C.c_float), _ptr(z, C.c_float),
+                _ptr(owner, C.c_int32), _ptr(calls, C.c_int32))
+        assert rc == 0, "reference fusedMM_csr returned %d" % rc
+        # the tuple adds val[j] * y[0] = row id once per edge: a second check that every edge ran once
+        deg = (pntre[:m].astype(np.int64) - pntrb[:m].astype(np.int64))
+        assert np.array_equal(calls[:m], deg), "the reference evaluated some edge zero or several times"
+        return owner[:m], calls[:m]
+
+
+def owners_from_ranges(rowb, rowe, m):
+    """Row -> thread id from the oracle's ranges [rowb[id], rowe[id]); -2 for a row in no range,
+    -3 for a row in two."""
+    own = np.full(m, -2, np.int64)
+    for t in range(len(rowb)):
+        b, e = int(rowb[t]), int(rowe[t])
+        if e > b:
+            own[b:e] = np.where(own[b:e] == -2, t, -3)
+    return own

@@ -118,3 +118,74 @@ def test_double_ops_against_reference(oracle_d, bits, t):
         oracle_d.opt(ot, g, X, Y, Z, beta=0.0, sop_kind=sk, mode=mode, V=4, L=8, S=8)
         tol = 2e-3 if t == "s" else 1e-13          # sigmoid: a table-bin flip; otherwise rounding
         assert np.abs(Z - want_t).max() <= tol * scale, (mode, np.abs(Z - want_t).max())
+
+
+def _rule(deg, nthreads, recompute=True, strict=True, tip_opens_next=True, restart=True):
+    """The partition rule with each of its steps switchable, used only to show
+    that the golden vectors tell the variants apart (all switches on = the rule
+    as the reference has it)."""
+    m = len(deg)
+    total = int(deg.sum())
+    quota = total // nthreads
+    own = np.zeros(m, np.int64)
+    cur = cum = 0
+    tt = 0
+    for i in range(m):
+        cum += int(deg[i])
+        cur += int(deg[i])
+        own[i] = tt
+        if (cur > quota if strict else cur >= quota) and tt + 1 < nthreads:
+            tt += 1
+            if tip_opens_next:
+                own[i] = tt
+            cur = 0 if restart else cur - quota
+            if recompute:
+                quota = (total - cum) // (nthreads - tt)
+    return own
+
+
+def _partition_golden():
+    d = np.load(os.path.join(GOLD, "partition.npz"))
+    for name in d["names"]:
+        name = str(name)
+        yield name, d[name + "_pntrb"], d[name + "_pntre"], int(d[name + "_m"]), \
+            {t: d["%s_owner_t%d" % (name, t)].astype(np.int64) for t in (2, 3, 5, 8, 16)}
+
+
+@pytest.mark.parametrize("bits", [32, 64])
+def test_partition_equals_the_reference_row_for_row(oracle, bits):
+    """orc_partition_rows against the thread the real reference (fusedMM.c:633-676,
+    -DPTTIME -DLOAD_BALANCE -DNTHREADS=t) was seen to evaluate every row on."""
+    from oracle_api import owners_from_ranges
+    it = np.int32 if bits == 32 else np.int64
+    checked = 0
+    for name, pb, pe, m, owners in _partition_golden():
+        for t, want in owners.items():
+            rc, rb, re = oracle.partition(pb.astype(it), pe.astype(it), t, m=m)
+            assert rc == 0, (name, t)
+            got = owners_from_ranges(rb, re, m)
+            assert got.min() >= 0, (name, t, "rows outside every range, or in two")
+            seen = want >= 0                       # rows with edges: the reference showed their thread
+            assert np.array_equal(got[seen], want[seen]), (name, t)
+            # ranges are contiguous and ascending, so rows without edges are pinned wherever
+            # they lie strictly between two rows of one thread
+            assert np.all(np.diff(got) >= 0), (name, t)
+            checked += int(seen.sum())
+    assert checked > 40000
+
+
+def test_partition_vectors_tell_the_rule_from_its_near_misses():
+    """Each plausible slip (quota never recomputed, >= for >, the tipping row
+    kept by the closing thread, the running count not restarted) disagrees with
+    the reference's recorded ownership on some case; the rule itself never does."""
+    variants = {"no_recompute": dict(recompute=False), "not_strict": dict(strict=False),
+                "tip_stays": dict(tip_opens_next=False), "no_restart": dict(restart=False)}
+    wrong = {v: 0 for v in variants}
+    for name, pb, pe, m, owners in _partition_golden():
+        deg = (pe - pb)[:m]
+        for t, want in owners.items():
+            seen = want >= 0
+            assert np.array_equal(_rule(deg, t)[seen], want[seen]), (name, t)
+            for v, kw in variants.items():
+                wrong[v] += int(not np.array_equal(_rule(deg, t, **kw)[seen], want[seen]))
+    assert all(n > 0 for n in wrong.values()), wrong

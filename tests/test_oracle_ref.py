@@ -71,3 +71,29 @@ def test_double_generic_path_bits(bits, t):
         assert od.generic(MSG[t], g, X, Y, B, sop_kind=sk) == 0
         assert np.array_equal(A.view(np.uint64), B.view(np.uint64))
     assert np.array_equal(od.table().view(np.uint64), Ref("sigmoid", bits, 64).table().view(np.uint64))
+
+
+@pytest.mark.parametrize("bits", [32, 64])
+@pytest.mark.parametrize("nthreads", [2, 3, 5, 8, 16])
+def test_partition_rows_live(oracle, bits, nthreads):
+    """orc_partition_rows against the thread the real reference (fusedMM.c:633-676 built
+    with -DPTTIME -DLOAD_BALANCE -DNTHREADS=n) is seen to evaluate each row on, for
+    fresh random skewed degree sets."""
+    from oracle_api import RefPartition, owners_from_ranges, ref_partition_available
+    if not ref_partition_available(nthreads, bits):
+        pytest.skip("oracle/_ref partition probe not built")
+    it = np.int32 if bits == 32 else np.int64
+    ref = RefPartition(nthreads, bits)
+    rng = np.random.default_rng(100 * nthreads + bits)
+    for rep in range(24):
+        n = int(rng.integers(1, 3000))
+        deg = np.minimum(rng.zipf(1.3 + 0.1 * (rep % 8), n), int(rng.integers(1, 1500)))
+        deg[rng.random(n) < 0.1 * (rep % 5)] = 0
+        ptr = np.concatenate([[0], np.cumsum(deg)]).astype(it)
+        m = n if rep % 3 else max(1, n // 2)
+        want, _ = ref.owners(ptr[:-1], ptr[1:], m)
+        rc, rb, re = oracle.partition(ptr[:-1], ptr[1:], nthreads, m=m)
+        assert rc == 0
+        got = owners_from_ranges(rb, re, m)
+        seen = want >= 0
+        assert got.min() >= 0 and np.array_equal(got[seen], want[seen]), (rep, n, m)
