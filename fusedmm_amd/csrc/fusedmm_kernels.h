@@ -255,6 +255,7 @@ __device__ __forceinline__ real_t sop_eval(int kind, real_t s, const real_t *tab
             int idx = (int)(((double)s + 5.0) * 204.8);
 #endif
             idx = idx > kSigmoidTableSize - 1 ? kSigmoidTableSize - 1 : idx;
+            idx = idx < 0 ? 0 : idx;   // only a NaN gets here (neither comparison above holds for it)
             t = tab[idx];
          }
          return (real_t)1.0 - t;   // single precision: exact in double for table values, one rounding either way
@@ -1050,13 +1051,15 @@ __global__ __launch_bounds__(kBlockThreads) void edge_scalar_kernel(const Params
       const IdxT je = wave_uniform<IdxT>(p.pntre[row]);
       Slice<R> xs;
       load_slice<V, L, R, EXACT>(xs, p.x + row * p.ldx, sl, p.k);
-      for (IdxT j0 = jb; j0 < je; j0 += S * U)
+      // slot numbers in 64 bits: an int32 slot next to 2^31 must not wrap when stepped past je
+      const int64_t je64 = (int64_t)je;
+      for (int64_t j0 = (int64_t)jb; j0 < je64; j0 += S * U)
       {
 #pragma unroll
          for (int u = 0; u < U; u++)
          {
-            const IdxT j = j0 + sub + u * S;
-            if (j < je)
+            const int64_t j = j0 + sub + u * S;
+            if (j < je64)
             {
                Slice<R> ys, t;
                load_slice<V, L, R, EXACT>(ys, p.y + (int64_t)p.indx[j] * p.ldy, sl, p.k);
@@ -1091,7 +1094,7 @@ __global__ __launch_bounds__(kBlockThreads) void validate_kernel(const Params<Id
    {
       const IdxT jb = p.pntrb[row], je = p.pntre[row];
       if (je < jb || jb < 0) { bad = true; continue; }
-      for (IdxT j = jb + lane; j < je; j += 64)
+      for (int64_t j = (int64_t)jb + lane; j < (int64_t)je; j += 64)   // 64-bit: no wrap next to 2^31
       {
          const IdxT c = p.indx[j];
          if (c < 0 || (int64_t)c >= n) bad = true;

@@ -120,10 +120,12 @@ def test_c2_graph_gcn_counts_degrees_and_spmm_is_linear(c2):
     assert torch.allclose(Zc, Za + Zb, rtol=1e-5, atol=2e-5)
 
 
-@pytest.mark.parametrize("name", ["c5", "c3"])
+@pytest.mark.parametrize("name", ["c5", "c3", "c4"])
 def test_skewed_full_size(oracle, name):
-    """Power-law (hubs of 10^6 neighbours) and R-MAT at full size: split rows,
-    determinism, beta rule, and oracle-checked windows including the longest row."""
+    """Power-law (hubs of 10^6 neighbours) and R-MAT (scale 22 at K=256, scale 24
+    at K=64 with 5.2e8 edges and int32 slot numbers up to 2^29) at full size:
+    split rows, determinism, beta rule, and oracle-checked windows including the
+    longest row and the last rows (the highest slot numbers)."""
     w = Resident(name)
     torch = w.torch
     m, k = w.g["rows"], w.k
@@ -134,10 +136,12 @@ def test_skewed_full_size(oracle, name):
     heavy_deg, _ = gpu_api.default_split(k)
     assert h == int((deg > heavy_deg).sum()) and s > h and o == 0
     hub = int(np.argmax(deg))
-    if name == "c5":
-        w.window_check(oracle, Z, hub, hub + 1)                      # 10^6 edges, 512 segments
+    if name in ("c5", "c4"):
+        w.window_check(oracle, Z, hub, hub + 1)                      # c5: 10^6 edges, 512 segments
     mid = m // 2
     w.window_check(oracle, Z, mid, mid + 256)
+    w.window_check(oracle, Z, 0, 8)                                  # R-MAT: the lowest row ids are the longest rows
+    w.window_check(oracle, Z, m - 256, m)
     Z2 = torch.full((m, k), 1.5, device=w.dev)
     w.call(Z2)
     assert torch.equal(Z, Z2)
