@@ -32,7 +32,8 @@ SOP_KIND_HOST, SOP_KIND_IDENTITY, SOP_KIND_SIGMOID, SOP_KIND_TDIST, SOP_KIND_FR,
 SUCCESS, FAIL, VOP_FAIL, ROP_FAIL, AOP_FAIL, SOP_FAIL, VSC_FAIL = 0, 1, 2, 4, 8, 16, 32
 NOT_ENOUGH_MEM, UNDEFINED_USER_FUNCTION, NO_OPT_IMPL = -1, 64, 128
 
-EXPORTS = ("fusedMM_csr", "fusedMM_csr_stream", "fusedMM_amd_index_bytes", "fusedMM_amd_value_bytes",
+EXPORTS = ("fusedMM_csr", "fusedMM_csr_stream", "fusedMM_csr_stream_noalloc", "fusedMM_amd_init",
+           "fusedMM_amd_noalloc_capacity", "fusedMM_amd_index_bytes", "fusedMM_amd_value_bytes",
            "fusedMM_amd_set_sop_kind", "fusedMM_amd_get_sop_kind", "fusedMM_amd_set_sop_callback",
            "fusedMM_amd_set_opt", "fusedMM_amd_set_validate", "fusedMM_amd_set_split", "fusedMM_amd_timing",
            "fusedMM_amd_timing_summary", "fusedMM_amd_timing_call", "fusedMM_amd_last_split", "fusedMM_amd_copy_probe",
@@ -66,6 +67,10 @@ def load(index_bits=32, value_bits=32):
     lib.fusedMM_csr.restype = C.c_int
     lib.fusedMM_csr_stream.argtypes = csr + [vp]
     lib.fusedMM_csr_stream.restype = C.c_int
+    lib.fusedMM_csr_stream_noalloc.argtypes = csr + [vp]
+    lib.fusedMM_csr_stream_noalloc.restype = C.c_int
+    lib.fusedMM_amd_init.restype = C.c_int
+    lib.fusedMM_amd_noalloc_capacity.restype = C.c_int64
     gf = lib.sgfusedMM_csr if value_bits == 32 else lib.dgfusedMM_csr   # kernels.h:17-37 of the reference
     gf.argtypes = [C.c_char] + csr[1:]
     gf.restype = None
@@ -107,13 +112,16 @@ def _addr(a):
 
 
 def fusedMM_csr(imessage, m, n, k, alpha, nnz, rows, cols, val, indx, pntrb, pntre, x, ldx, y, ldy, beta, z, ldz,
-                index_bits=32, stream=None, value_bits=32):
+                index_bits=32, stream=None, value_bits=32, noalloc=False):
     """Same argument list as the C entry point (include/fusedMM.h).  Operands
     are numpy arrays (host memory) or torch tensors / integer addresses (device
-    memory).  With `stream` (an integer hipStream_t) the call is asynchronous."""
+    memory).  With `stream` (an integer hipStream_t) the call is asynchronous;
+    noalloc=True takes the entry point that allocates nothing."""
     lib = load(index_bits, value_bits)
     args = [imessage, m, n, k, alpha, nnz, rows, cols, _addr(val), _addr(indx), _addr(pntrb), _addr(pntre),
             _addr(x), ldx, _addr(y), ldy, beta, _addr(z), ldz]
+    if noalloc:
+        return lib.fusedMM_csr_stream_noalloc(*args, stream)
     if stream is None:
         return lib.fusedMM_csr(*args)
     return lib.fusedMM_csr_stream(*args, stream)

@@ -29,6 +29,15 @@
 #include "../../include/fusedmm_amd.h"
 #include "fusedmm_kernels.h"
 
+// Device memory of the entry point that allocates nothing (fusedMM_csr_stream_noalloc):
+// the sigmoid table, the queue and claim counters, the queued-row bitmap, the
+// heavy-row queue, the segment descriptors and the partial results of split rows,
+// carved out of this array call by call.  Every GPU the library runs on holds its
+// own copy until the process ends.  In host code the name is only a handle: the
+// address kernels and copies use comes from hipGetSymbolAddress, once per device.
+#define FUSEDMM_AMD_SCRATCH_BYTES (32u << 20)
+static __device__ __align__(256) unsigned char fmm_scratch[FUSEDMM_AMD_SCRATCH_BYTES];
+
 namespace {
 
 using namespace fmm;
@@ -65,13 +74,26 @@ struct Buffer {
    size_t bytes = 0;
 };
 
+// The two sets of work queues a GPU can hold: buffers that grow with the
+// largest call seen (every ordinary entry point), and the fixed static array.
+enum : int { kQueuesGrown = 0, kQueuesStatic = 1 };
+
 struct DeviceState {
-   bool ready = false;
+   bool basics = false;       // num_cu and the ordering events
+   bool ready = false;        // allocated table and counters of the ordinary entry points
    int num_cu = 0;
    val_t *sigmoid_table = nullptr;
    Counters *ctr = nullptr;
    Buffer heavy, segs, partial, queued;
    Buffer stage[8];           // host-pointer mode: pntrb, pntre, indx, val, x, y, z, spare
+   // the static array of this device (address from hipGetSymbolAddress), once set up
+   unsigned char *scratch = nullptr;
+   // Calls that share a set of queues must not overlap: each call records order_ev
+   // behind its last kernel, and a call on another stream first waits for it.
+   hipEvent_t order_ev[2];
+   hipStream_t last_stream[2] = {nullptr, nullptr};
+   bool pending[2] = {false, false};
+   Counters *last_ctr = nullptr;   // counters of the most recent call (fusedMM_amd_last_split)
    // timing
    hipEvent_t ev[kTimingSlots][4];
    bool ev_made = false;
@@ -144,9 +166,19 @@ void build_sigmoid_table(val_t *t)
    }
 }
 
-int grow(Buffer &b, size_t bytes)
+// `capturing`: the call is being recorded into a HIP graph.  Replacing a buffer
+// then would leave the graph (and any graph captured earlier) with the address
+// of freed memory, so the call is refused instead.
+int grow(Buffer &b, size_t bytes, bool capturing = false)
 {
    if (bytes <= b.bytes) return FUSEDMM_SUCCESS_RETURN;
+   if (capturing)
+   {
+      FMM_LOG("a work buffer would have to grow (%zu -> %zu bytes) while the stream is being captured; "
+              "run one call of this size outside the capture first, or use fusedMM_csr_stream_noalloc",
+              b.bytes, bytes);
+      return FUSEDMM_NOT_ENOUGH_MEM;
+   }
    if (b.ptr) FMM_HIP(hipFree(b.ptr));
    b.ptr = nullptr;
    b.bytes = 0;
@@ -155,17 +187,33 @@ int grow(Buffer &b, size_t bytes)
    return FUSEDMM_SUCCESS_RETURN;
 }
 
-int device_state(DeviceState **out)
+// What every entry point needs of the current device; allocates no device memory.
+int device_basics(DeviceState **out)
 {
    int dev = 0;
    FMM_HIP(hipGetDevice(&dev));
    if (dev < 0 || dev >= kMaxDevices) return FUSEDMM_FAIL_RETURN;
    DeviceState &d = g.dev[dev];
+   if (!d.basics)
+   {
+      int cus = 0;
+      FMM_HIP(hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev));
+      d.num_cu = cus > 0 ? cus : 256;
+      for (int q = 0; q < 2; q++) FMM_HIP(hipEventCreateWithFlags(&d.order_ev[q], hipEventDisableTiming));
+      d.basics = true;
+   }
+   *out = &d;
+   return FUSEDMM_SUCCESS_RETURN;
+}
+
+int device_state(DeviceState **out)
+{
+   DeviceState *dp = nullptr;
+   int st0 = device_basics(&dp);
+   if (st0) return st0;
+   DeviceState &d = *dp;
    if (!d.ready)
    {
-      hipDeviceProp_t prop;
-      FMM_HIP(hipGetDeviceProperties(&prop, dev));
-      d.num_cu = prop.multiProcessorCount > 0 ? prop.multiProcessorCount : 256;
       val_t host_tab[kSigmoidTableSize];
       build_sigmoid_table(host_tab);
       FMM_HIP(hipMalloc((void **)&d.sigmoid_table, sizeof(host_tab)));
@@ -175,6 +223,28 @@ int device_state(DeviceState **out)
       d.ready = true;
    }
    *out = &d;
+   return FUSEDMM_SUCCESS_RETURN;
+}
+
+// ---- the static array: fixed head, then the queues of the call in progress ----------
+constexpr size_t align256(size_t v) { return (v + 255u) & ~(size_t)255u; }
+constexpr size_t kScratchTableOff = 0;
+constexpr size_t kScratchCtrOff = align256(kSigmoidTableSize * sizeof(val_t));
+constexpr size_t kScratchQueuesOff = kScratchCtrOff + align256(sizeof(Counters));
+
+// Once per device, with that device current: find this device's copy of the
+// array, put the sigmoid table at its head and zero the counters.
+int scratch_setup(DeviceState &d)
+{
+   if (d.scratch) return FUSEDMM_SUCCESS_RETURN;
+   unsigned char *base = nullptr;
+   FMM_HIP(hipGetSymbolAddress((void **)&base, HIP_SYMBOL(fmm_scratch)));
+   if (!base) return FUSEDMM_FAIL_RETURN;
+   val_t host_tab[kSigmoidTableSize];
+   build_sigmoid_table(host_tab);
+   FMM_HIP(hipMemcpy(base + kScratchTableOff, host_tab, sizeof(host_tab), hipMemcpyHostToDevice));
+   FMM_HIP(hipMemset(base + kScratchCtrOff, 0, sizeof(Counters)));
+   d.scratch = base;
    return FUSEDMM_SUCCESS_RETURN;
 }
 
@@ -340,11 +410,27 @@ struct Args {
    val_t beta;
 };
 
-int run_on_device(const Args &a, const Plan &pl, int sop_kind, hipStream_t stream);
+int run_on_device(const Args &a, const Plan &pl, int sop_kind, hipStream_t stream, int queues = kQueuesGrown);
+int validate_host_pointers(const Args &h);
+int validate_operands(const Args &a, hipStream_t stream, int queues = kQueuesGrown);
+
+// Is `stream` being recorded into a HIP graph?  The legacy default stream cannot be.
+int stream_capturing(hipStream_t stream, bool *capturing)
+{
+   *capturing = false;
+   if (!stream) return FUSEDMM_SUCCESS_RETURN;
+   hipStreamCaptureStatus cs = hipStreamCaptureStatusNone;
+   FMM_HIP(hipStreamIsCapturing(stream, &cs));
+   *capturing = (cs != hipStreamCaptureStatusNone);
+   return FUSEDMM_SUCCESS_RETURN;
+}
 
 // One call of the kernels, k <= kMaxK.  Everything here is device memory.
-// Enqueues on `stream`, does not wait.
-int run_slab(const Args &a, const Plan &pl, int sop_kind, hipStream_t stream)
+// Enqueues on `stream`, does not wait.  `queues` says where the call's work
+// queues live: kQueuesGrown (allocated, grown to the largest call seen) or
+// kQueuesStatic (carved out of the static array; the call is refused when they
+// do not fit, and nothing is allocated).
+int run_slab(const Args &a, const Plan &pl, int sop_kind, hipStream_t stream, int queues)
 {
    if (a.m <= 0) return FUSEDMM_SUCCESS_RETURN;
    if (a.k < 1) return FUSEDMM_SUCCESS_RETURN;
@@ -364,7 +450,11 @@ int run_slab(const Args &a, const Plan &pl, int sop_kind, hipStream_t stream)
       return FUSEDMM_FAIL_RETURN;
    }
    DeviceState *d = nullptr;
-   int st = device_state(&d);
+   int st = (queues == kQueuesStatic) ? device_basics(&d) : device_state(&d);
+   if (st) return st;
+   if (queues == kQueuesStatic) { st = scratch_setup(*d); if (st) return st; }
+   bool capturing = false;
+   st = stream_capturing(stream, &capturing);
    if (st) return st;
 
    // 16-byte accesses need 16-byte aligned rows: leading dimensions a multiple of 4 floats / 2 doubles
@@ -385,7 +475,6 @@ int run_slab(const Args &a, const Plan &pl, int sop_kind, hipStream_t stream)
    p.beta_zero = (pl.opt_rule && a.beta == 0.0f) ? 1 : 0;
    p.sop_kind = sop_kind;
    p.imessage = a.imessage;
-   p.sigmoid_table = d->sigmoid_table;
 
    // heavy-row split: segments of about 1 MiB of gathered rows but at most 2048 edges
    // (measured best on the R-MAT and power-law benchmark graphs: shorter segments pay
@@ -410,24 +499,60 @@ int run_slab(const Args &a, const Plan &pl, int sop_kind, hipStream_t stream)
    if (cap_seg * p.kpad * (int64_t)kValBytes > max_partial_bytes) cap_seg = max_partial_bytes / (p.kpad * (int64_t)kValBytes);
    if (cap_seg > 0x7FFFFFFF) cap_seg = 0x7FFFFFFF;
    if (cap_heavy > 0x7FFFFFFF) cap_heavy = 0x7FFFFFFF;
-   st = grow(d->heavy, (size_t)cap_heavy * sizeof(HeavyRow)); if (st) return st;
-   st = grow(d->segs, (size_t)cap_seg * sizeof(SegDesc)); if (st) return st;
-   st = grow(d->partial, (size_t)cap_seg * p.kpad * kValBytes); if (st) return st;
    const int64_t queued_words = (a.m + 31) / 32;
-   st = grow(d->queued, (size_t)queued_words * sizeof(unsigned int)); if (st) return st;
-   p.ctr = d->ctr;
-   p.heavy = (HeavyRow *)d->heavy.ptr;
-   p.segs = (SegDesc *)d->segs.ptr;
-   p.partial = (val_t *)d->partial.ptr;
-   p.queued = (unsigned int *)d->queued.ptr;
+   const size_t b_heavy = (size_t)cap_heavy * sizeof(HeavyRow), b_segs = (size_t)cap_seg * sizeof(SegDesc),
+                b_partial = (size_t)cap_seg * p.kpad * kValBytes, b_queued = (size_t)queued_words * sizeof(unsigned int);
+   if (queues == kQueuesStatic)
+   {
+      // same capacities as the allocating entry points (so the same rows are split and
+      // the results are the same bits), laid out behind the fixed head of the array
+      const size_t o_queued = kScratchQueuesOff, o_heavy = o_queued + align256(b_queued),
+                   o_segs = o_heavy + align256(b_heavy), o_partial = o_segs + align256(b_segs),
+                   end = o_partial + align256(b_partial);
+      if (end > (size_t)FUSEDMM_AMD_SCRATCH_BYTES)
+      {
+         FMM_LOG("fusedMM_csr_stream_noalloc: m=%lld, nnz=%lld, k=%lld need %zu bytes of work queues; the static "
+                 "array holds %zu (use fusedMM_csr_stream for this size)",
+                 (long long)a.m, (long long)nnz_hint, (long long)a.k, end, (size_t)FUSEDMM_AMD_SCRATCH_BYTES);
+         return FUSEDMM_NOT_ENOUGH_MEM;
+      }
+      unsigned char *base = d->scratch;   // this device's address, never the array's name
+      p.sigmoid_table = (const val_t *)(base + kScratchTableOff);
+      p.ctr = (Counters *)(base + kScratchCtrOff);
+      p.queued = (unsigned int *)(base + o_queued);
+      p.heavy = (HeavyRow *)(base + o_heavy);
+      p.segs = (SegDesc *)(base + o_segs);
+      p.partial = (val_t *)(base + o_partial);
+   }
+   else
+   {
+      st = grow(d->heavy, b_heavy, capturing); if (st) return st;
+      st = grow(d->segs, b_segs, capturing); if (st) return st;
+      st = grow(d->partial, b_partial, capturing); if (st) return st;
+      st = grow(d->queued, b_queued, capturing); if (st) return st;
+      p.sigmoid_table = d->sigmoid_table;
+      p.ctr = d->ctr;
+      p.heavy = (HeavyRow *)d->heavy.ptr;
+      p.segs = (SegDesc *)d->segs.ptr;
+      p.partial = (val_t *)d->partial.ptr;
+      p.queued = (unsigned int *)d->queued.ptr;
+   }
    p.cap_heavy = (unsigned int)cap_heavy;
    p.cap_seg = (unsigned int)cap_seg;
+   d->last_ctr = p.ctr;
+
+   // Calls that share these queues must run one after the other.  On one stream
+   // they do; a call on another stream first waits for the previous call's last
+   // kernel.  (Not while capturing: an event recorded into a graph cannot be
+   // waited on from outside it; the graph's launches are ordered by their stream.)
+   if (!capturing && d->pending[queues] && d->last_stream[queues] != stream)
+      FMM_HIP(hipStreamWaitEvent(stream, d->order_ev[queues], 0));
 
    {
       int64_t rb = (queued_words + kBlockThreads - 1) / kBlockThreads;
       if (rb > (int64_t)d->num_cu * 4) rb = (int64_t)d->num_cu * 4;
       if (rb < 1) rb = 1;
-      hipLaunchKernelGGL(reset_kernel, dim3((unsigned int)rb), dim3(kBlockThreads), 0, stream, d->ctr, p.queued, queued_words);
+      hipLaunchKernelGGL(reset_kernel, dim3((unsigned int)rb), dim3(kBlockThreads), 0, stream, p.ctr, p.queued, queued_words);
    }
 
    Launch l;
@@ -436,7 +561,7 @@ int run_slab(const Args &a, const Plan &pl, int sop_kind, hipStream_t stream)
    l.nnz_hint = nnz_hint;
    l.stream = stream;
    l.ev = nullptr;
-   if (g.timing && g.timing_calls < kTimingSlots)
+   if (g.timing && g.timing_calls < kTimingSlots && queues == kQueuesGrown && !capturing)
    {
       if (!d->ev_made)
       {
@@ -450,17 +575,27 @@ int run_slab(const Args &a, const Plan &pl, int sop_kind, hipStream_t stream)
 
    switch (pl.op)
    {
-      case OP_GCN: return launch_op<OP_GCN, -1>(p, sh, l);
-      case OP_SPMM: return launch_op<OP_SPMM, -1>(p, sh, l);
+      case OP_GCN: st = launch_op<OP_GCN, -1>(p, sh, l); break;
+      case OP_SPMM: st = launch_op<OP_SPMM, -1>(p, sh, l); break;
       case OP_DOT:
-         if (sop_kind == SOP_SIGMOID) return launch_op<OP_DOT, SOP_SIGMOID>(p, sh, l);
-         return launch_op<OP_DOT, -1>(p, sh, l);
+         if (sop_kind == SOP_SIGMOID) st = launch_op<OP_DOT, SOP_SIGMOID>(p, sh, l);
+         else st = launch_op<OP_DOT, -1>(p, sh, l);
+         break;
       case OP_DIST:
-         if (sop_kind == SOP_TDIST) return launch_op<OP_DIST, SOP_TDIST>(p, sh, l);
-         if (sop_kind == SOP_FR) return launch_op<OP_DIST, SOP_FR>(p, sh, l);
-         return launch_op<OP_DIST, -1>(p, sh, l);
-      default: return launch_op<OP_GENERIC, -1>(p, sh, l);
+         if (sop_kind == SOP_TDIST) st = launch_op<OP_DIST, SOP_TDIST>(p, sh, l);
+         else if (sop_kind == SOP_FR) st = launch_op<OP_DIST, SOP_FR>(p, sh, l);
+         else st = launch_op<OP_DIST, -1>(p, sh, l);
+         break;
+      default: st = launch_op<OP_GENERIC, -1>(p, sh, l); break;
    }
+   if (st) return st;
+   if (!capturing)
+   {
+      FMM_HIP(hipEventRecord(d->order_ev[queues], stream));
+      d->pending[queues] = true;
+      d->last_stream[queues] = stream;
+   }
+   return FUSEDMM_SUCCESS_RETURN;
 }
 
 bool is_device_pointer(const void *p)
@@ -502,9 +637,24 @@ int operand_residence(const Args &a)
 int stage_up(const Args &h, const Plan &pl, Args *a, int64_t *slots_out)
 {
    if (h.n <= 0) { FMM_LOG("n (rows of Y) must be positive for host operands"); return FUSEDMM_FAIL_RETURN; }
+   if (h.ldy < h.k || h.ldz < h.k || (pl.reads_x && h.ldx < h.k))
+   {
+      FMM_LOG("leading dimension smaller than k");
+      return FUSEDMM_FAIL_RETURN;
+   }
+   if (!h.indx || !h.pntrb || !h.pntre || !h.y || !h.z || (pl.reads_x && !h.x))
+   {
+      FMM_LOG("NULL operand");
+      return FUSEDMM_FAIL_RETURN;
+   }
    DeviceState *d = nullptr;
    int st = device_state(&d);
    if (st) return st;
+   if (g.validate)
+   {
+      st = validate_host_pointers(h);
+      if (st) return st;
+   }
    int64_t slots = 0;
    for (int64_t i = 0; i < h.m; i++)
       if ((int64_t)h.pntre[i] > slots) slots = (int64_t)h.pntre[i];
@@ -529,8 +679,10 @@ int stage_up(const Args &h, const Plan &pl, Args *a, int64_t *slots_out)
    FMM_HIP(hipMemcpyAsync(d->stage[1].ptr, h.pntre, b_ptr, hipMemcpyHostToDevice, s));
    if (slots > 0) FMM_HIP(hipMemcpyAsync(d->stage[2].ptr, h.indx, (size_t)slots * sizeof(idx_t), hipMemcpyHostToDevice, s));
    if (need_val && slots > 0) FMM_HIP(hipMemcpyAsync(d->stage[3].ptr, h.val, (size_t)slots * kValBytes, hipMemcpyHostToDevice, s));
-   if (pl.reads_x) FMM_HIP(hipMemcpyAsync(d->stage[4].ptr, h.x, b_x, hipMemcpyHostToDevice, s));
-   FMM_HIP(hipMemcpyAsync(d->stage[5].ptr, h.y, b_y, hipMemcpyHostToDevice, s));
+   // the caller's arrays need not extend past the last element the reference reads:
+   // (rows - 1) * ld + k elements, not rows * ld
+   if (pl.reads_x) FMM_HIP(hipMemcpyAsync(d->stage[4].ptr, h.x, b_x - (size_t)(h.ldx - h.k) * kValBytes, hipMemcpyHostToDevice, s));
+   FMM_HIP(hipMemcpyAsync(d->stage[5].ptr, h.y, b_y - (size_t)(h.ldy - h.k) * kValBytes, hipMemcpyHostToDevice, s));
    const bool overwrite = pl.opt_rule && h.beta == 0.0f;
    if (!overwrite)   // one contiguous copy, padding columns included (they are never written back)
       FMM_HIP(hipMemcpyAsync(d->stage[6].ptr, h.z, b_z - (size_t)(h.ldz - h.k) * kValBytes, hipMemcpyHostToDevice, s));
@@ -576,6 +728,11 @@ int run_staged(const Args &h, const Plan &pl, int sop_kind)
    int64_t slots = 0;
    int st = stage_up(h, pl, &a, &slots);
    if (st) return st;
+   if (g.validate)
+   {
+      st = validate_operands(a, 0);
+      if (st) return st;
+   }
    st = run_on_device(a, pl, sop_kind, 0);
    if (st) return st;
    return stage_down(h, a);
@@ -630,7 +787,7 @@ int edge_scalars(const Args &a, val_t *d_s, DeviceState *d, hipStream_t stream)
 // FUSEDMM_VALIDATE=1 / fusedMM_amd_set_validate(1): check row pointers and
 // column ids on the device before any kernel dereferences them.  Costs a pass
 // over the CSR arrays and a synchronisation per call.
-int validate_operands(const Args &a, hipStream_t stream)
+int validate_operands(const Args &a, hipStream_t stream, int queues)
 {
    if (a.n <= 0 || !a.indx || !a.pntrb || !a.pntre)
    {
@@ -638,12 +795,16 @@ int validate_operands(const Args &a, hipStream_t stream)
       return FUSEDMM_FAIL_RETURN;
    }
    DeviceState *d = nullptr;
-   int st = device_state(&d);
+   int st = (queues == kQueuesStatic) ? device_basics(&d) : device_state(&d);
    if (st) return st;
+   if (queues == kQueuesStatic) { st = scratch_setup(*d); if (st) return st; }
+   Counters *ctr = (queues == kQueuesStatic) ? (Counters *)(d->scratch + kScratchCtrOff) : d->ctr;
    Params<idx_t> p;
    memset(&p, 0, sizeof(p));
    p.pntrb = a.pntrb; p.pntre = a.pntre; p.indx = a.indx; p.m = a.m;
-   unsigned int *flag = &d->ctr->invalid;
+   // the flag is one of the shared counters: wait for a call still using them on another stream
+   if (d->pending[queues] && d->last_stream[queues] != stream) FMM_HIP(hipStreamWaitEvent(stream, d->order_ev[queues], 0));
+   unsigned int *flag = &ctr->invalid;
    FMM_HIP(hipMemsetAsync(flag, 0, sizeof(unsigned int), stream));
    int64_t blocks = (a.m + kWavesPerBlock - 1) / kWavesPerBlock;
    if (blocks > (int64_t)d->num_cu * 8) blocks = (int64_t)d->num_cu * 8;
@@ -658,6 +819,25 @@ int validate_operands(const Args &a, hipStream_t stream)
    }
    return FUSEDMM_SUCCESS_RETURN;
 }
+
+// The same check for row pointers that are host memory, before anything is sized from them.
+int validate_host_pointers_of(const Args &h, const idx_t *pb, const idx_t *pe)
+{
+   if (!pb || !pe)
+   {
+      FMM_LOG("operand check: NULL row pointers");
+      return FUSEDMM_FAIL_RETURN;
+   }
+   for (int64_t i = 0; i < h.m; i++)
+      if (pb[i] < 0 || pe[i] < pb[i])
+      {
+         FMM_LOG("operand check failed: row %lld has pntrb=%lld, pntre=%lld", (long long)i, (long long)pb[i],
+                 (long long)pe[i]);
+         return FUSEDMM_FAIL_RETURN;
+      }
+   return FUSEDMM_SUCCESS_RETURN;
+}
+int validate_host_pointers(const Args &h) { return validate_host_pointers_of(h, h.pntrb, h.pntre); }
 
 int64_t max_slot(const idx_t *h_pe, int64_t m)
 {
@@ -716,15 +896,16 @@ int run_wide_reduction(const Args &a, const Plan &pl, int sop_kind)
 
 // Everything here is device memory.  Enqueues on `stream`, does not wait
 // (except for wide rows with a whole-row reduction, see run_wide_reduction).
-int run_on_device(const Args &a, const Plan &pl, int sop_kind, hipStream_t stream)
+int run_on_device(const Args &a, const Plan &pl, int sop_kind, hipStream_t stream, int queues)
 {
    if (a.m <= 0 || a.k < 1) return FUSEDMM_SUCCESS_RETURN;
-   if (g.validate)
+   if (a.k <= kMaxK) return run_slab(a, pl, sop_kind, stream, queues);
+   if (queues == kQueuesStatic)
    {
-      int st = validate_operands(a, stream);
-      if (st) return st;
+      FMM_LOG("fusedMM_csr_stream_noalloc: k=%lld is beyond the %d columns one kernel instance holds "
+              "(use fusedMM_csr_stream)", (long long)a.k, kMaxK);
+      return FUSEDMM_NOT_ENOUGH_MEM;
    }
-   if (a.k <= kMaxK) return run_slab(a, pl, sop_kind, stream);
    if (a.ldy < a.k || a.ldz < a.k || (pl.reads_x && a.ldx < a.k))
    {
       FMM_LOG("leading dimension smaller than k");
@@ -740,7 +921,7 @@ int run_on_device(const Args &a, const Plan &pl, int sop_kind, hipStream_t strea
          s.x = a.x ? a.x + off : nullptr;
          s.y = a.y + off;
          s.z = a.z + off;
-         int st = run_slab(s, pl, sop_kind, stream);
+         int st = run_slab(s, pl, sop_kind, stream, queues);
          if (st) return st;
       }
       return FUSEDMM_SUCCESS_RETURN;
@@ -760,6 +941,13 @@ int run_host_sop(const Args &a, const idx_t *h_pb, const idx_t *h_pe, int64_t sl
    DeviceState *d = nullptr;
    int st = device_state(&d);
    if (st) return st;
+   if (g.validate)   // before pass 1 dereferences a column id, and before the host indexes by the row pointers
+   {
+      st = validate_host_pointers_of(a, h_pb, h_pe);
+      if (st) return st;
+      st = validate_operands(a, 0);
+      if (st) return st;
+   }
    const bool overwrite = pl.opt_rule && a.beta == 0.0f;
    if (overwrite)
       hipLaunchKernelGGL(zero_rows_kernel, dim3((unsigned int)(d->num_cu * 8)), dim3(kBlockThreads), 0, 0, a.z, a.m, a.k, a.ldz);
@@ -807,7 +995,7 @@ fusedMM_amd_sop_fn host_sop_function()
    return (fusedMM_amd_sop_fn)dlsym(RTLD_DEFAULT, "SOP_UDEF_FUNC");
 }
 
-int entry(const Args &a, bool async, hipStream_t stream)
+int entry(const Args &a, bool async, hipStream_t stream, int queues = kQueuesGrown)
 {
    std::lock_guard<std::mutex> lock(g.mu);
    read_env_once();
@@ -854,12 +1042,26 @@ int entry(const Args &a, bool async, hipStream_t stream)
          return stage_down(a, dv);
       }
    }
-   if (async) return run_on_device(a, pl, sop_kind, stream);
+   if (async)
+   {
+      if (a.m <= 0 || a.k < 1) return FUSEDMM_SUCCESS_RETURN;
+      if (g.validate)
+      {
+         st = validate_operands(a, stream, queues);
+         if (st) return st;
+      }
+      return run_on_device(a, pl, sop_kind, stream, queues);
+   }
    if (a.m <= 0 || a.k < 1) return FUSEDMM_SUCCESS_RETURN;
    const int where = operand_residence(a);
    if (where < 0) return FUSEDMM_FAIL_RETURN;
    if (where == 1)
    {
+      if (g.validate)
+      {
+         st = validate_operands(a, 0);
+         if (st) return st;
+      }
       st = run_on_device(a, pl, sop_kind, 0);
       if (st) return st;
       return hip_status(hipStreamSynchronize(0), "hipStreamSynchronize");
@@ -895,6 +1097,30 @@ int fusedMM_csr_stream(const int32_t imessage, const INDEXTYPE m, const INDEXTYP
              (int64_t)ldx, (int64_t)ldy, (int64_t)ldz, beta};
    return entry(a, true, (hipStream_t)stream);
 }
+
+int fusedMM_csr_stream_noalloc(const int32_t imessage, const INDEXTYPE m, const INDEXTYPE n, const INDEXTYPE k,
+                               const VALUETYPE alpha, const INDEXTYPE nnz, const INDEXTYPE rows, const INDEXTYPE cols,
+                               const VALUETYPE *val, const INDEXTYPE *indx, const INDEXTYPE *pntrb, const INDEXTYPE *pntre,
+                               const VALUETYPE *x, const INDEXTYPE ldx, const VALUETYPE *y, const INDEXTYPE ldy,
+                               const VALUETYPE beta, VALUETYPE *z, const INDEXTYPE ldz, void *stream)
+{
+   (void)alpha; (void)rows; (void)cols;
+   Args a = {imessage, (int64_t)m, (int64_t)n, (int64_t)k, (int64_t)nnz, val, indx, pntrb, pntre, x, y, z,
+             (int64_t)ldx, (int64_t)ldy, (int64_t)ldz, beta};
+   return entry(a, true, (hipStream_t)stream, kQueuesStatic);
+}
+
+int fusedMM_amd_init(void)
+{
+   std::lock_guard<std::mutex> lock(g.mu);
+   read_env_once();
+   DeviceState *d = nullptr;
+   int st = device_state(&d);
+   if (st) return st;
+   return scratch_setup(*d);
+}
+
+int64_t fusedMM_amd_noalloc_capacity(void) { return (int64_t)FUSEDMM_AMD_SCRATCH_BYTES; }
 
 #ifdef FMM_DOUBLE
 #define FMM_GFUSEDMM dgfusedMM_csr
@@ -1022,11 +1248,12 @@ int fusedMM_amd_last_split(unsigned int *heavy_rows, unsigned int *segments, uns
 {
    std::lock_guard<std::mutex> lock(g.mu);
    DeviceState *d = nullptr;
-   int st = device_state(&d);
+   int st = device_basics(&d);
    if (st) return st;
    Counters c;
+   memset(&c, 0, sizeof(c));
    FMM_HIP(hipDeviceSynchronize());
-   FMM_HIP(hipMemcpy(&c, d->ctr, sizeof(c), hipMemcpyDeviceToHost));
+   if (d->last_ctr) FMM_HIP(hipMemcpy(&c, d->last_ctr, sizeof(c), hipMemcpyDeviceToHost));
    if (heavy_rows) *heavy_rows = c.n_heavy;
    if (segments) *segments = c.n_seg;
    if (overflow) *overflow = c.overflow;
@@ -1053,11 +1280,12 @@ void fusedMM_amd_finalize(void)
    for (int dev = 0; dev < kMaxDevices; dev++)
    {
       DeviceState &d = g.dev[dev];
-      if (!d.ready) continue;
+      if (!d.basics) continue;
       if (hipSetDevice(dev) != hipSuccess) continue;
       (void)hipDeviceSynchronize();
-      (void)hipFree(d.sigmoid_table);
-      (void)hipFree(d.ctr);
+      for (int q = 0; q < 2; q++) (void)hipEventDestroy(d.order_ev[q]);
+      if (d.sigmoid_table) (void)hipFree(d.sigmoid_table);
+      if (d.ctr) (void)hipFree(d.ctr);
       Buffer *bufs[] = {&d.heavy, &d.segs, &d.partial, &d.queued};
       for (Buffer *b : bufs) { if (b->ptr) (void)hipFree(b->ptr); *b = Buffer(); }
       for (Buffer &b : d.stage) { if (b.ptr) (void)hipFree(b.ptr); b = Buffer(); }

@@ -50,8 +50,13 @@ void fusedMM_amd_set_sop_callback(fusedMM_amd_sop_fn fn);
  * the call returns without waiting.  No counterpart in the reference; it is what
  * a framework that already keeps its tensors on the GPU binds (the reference's
  * CMakeLists.txt:1-14 packages fusedMM_csr for DGL).  Every call on a GPU uses
- * that GPU's one set of work queues: calls enqueued on different streams must
- * not overlap in time (use one stream, or order them with events).
+ * that GPU's one set of work queues, so the library runs calls enqueued on
+ * different streams one after the other (each waits for the previous call's last
+ * kernel).  Under HIP graph capture that ordering is the caller's, and a call
+ * whose work queues would have to grow returns FUSEDMM_NOT_ENOUGH_MEM: run one
+ * call of the same size before capturing; a later, larger call re-allocates the
+ * queues and invalidates graphs captured earlier (fusedMM_csr_stream_noalloc has
+ * neither restriction).
  * FUSEDMM_SOP_KIND_HOST is
  * not available here (it needs the host between passes): returns
  * FUSEDMM_UNDEFINED_USER_FUNCTION.
@@ -64,6 +69,41 @@ int fusedMM_csr_stream
    const VALUETYPE *x, const INDEXTYPE ldx, const VALUETYPE *y, const INDEXTYPE ldy,
    const VALUETYPE beta, VALUETYPE *z, const INDEXTYPE ldz, void *stream
 );
+
+/*
+ * fusedMM_csr_stream for callers that cannot allocate device memory: code under
+ * HIP graph capture, tight serving loops, harnesses that forbid hipMalloc.  No
+ * counterpart in the reference.  Same arguments, results (bit for bit) and rules
+ * as fusedMM_csr_stream, but the call's work queues (counters, queued-row bitmap,
+ * heavy-row queue, segment descriptors, partial results of split rows) and the
+ * sigmoid table live in a static device array of fusedMM_amd_noalloc_capacity()
+ * bytes (32 MiB) that every GPU the library runs on holds until the process ends;
+ * the call allocates and frees nothing.  A call whose queues, sized from m, nnz
+ * and k exactly as fusedMM_csr_stream sizes them, do not fit returns
+ * FUSEDMM_NOT_ENOUGH_MEM with a message on stderr and touches nothing; so does
+ * k > 2048.  (The sigmoid benchmark at K=128 with 2^20 rows and 2^24 edges needs
+ * 7.4 MiB.)  Pass the true nnz: it sizes the queues.  The first call on a device
+ * looks up the array's address and copies the 2048-entry table there; do that
+ * ahead of time, outside any capture, with fusedMM_amd_init().  All calls on a
+ * GPU share the one array: calls enqueued on different streams are ordered one
+ * after the other by the library, except while a stream is being captured, where
+ * the caller must keep them from overlapping.
+ */
+int fusedMM_csr_stream_noalloc
+(
+   const int32_t imessage, const INDEXTYPE m, const INDEXTYPE n, const INDEXTYPE k,
+   const VALUETYPE alpha, const INDEXTYPE nnz, const INDEXTYPE rows, const INDEXTYPE cols,
+   const VALUETYPE *val, const INDEXTYPE *indx, const INDEXTYPE *pntrb, const INDEXTYPE *pntre,
+   const VALUETYPE *x, const INDEXTYPE ldx, const VALUETYPE *y, const INDEXTYPE ldy,
+   const VALUETYPE beta, VALUETYPE *z, const INDEXTYPE ldz, void *stream
+);
+int64_t fusedMM_amd_noalloc_capacity(void);
+
+/* Set up the current device ahead of the first call: small fixed allocations of
+ * the ordinary entry points (sigmoid table, counters) and the static array of
+ * fusedMM_csr_stream_noalloc.  Optional; every entry point does its part of this
+ * on first use.  Returns a fusedMM status code. */
+int fusedMM_amd_init(void);
 
 /*
  * The reference's second-level entry (kernels/include/kernels.h:32-37,
