@@ -1,0 +1,252 @@
+"""Entry points and switches around fusedMM_csr: the reference's second-level
+entry sgfusedMM_csr / dgfusedMM_csr (kernels/src/kernels.c:456-631), the device
+copy of the sigmoid table, the operand check on every path, calls on several
+streams, and inputs at the edge of what the reference defines."""
+import ctypes as C
+
+import numpy as np
+import pytest
+
+import fusedmm_amd as fa
+import gpu_api
+import graphs
+from oracle_api import MSG, SOP_NAMES
+
+pytestmark = pytest.mark.gpu
+GOLD = __import__("os").path.join(__import__("os").path.dirname(__import__("os").path.abspath(__file__)), "golden")
+
+
+def _dev(a):
+    import torch
+    return None if a is None else torch.from_numpy(np.ascontiguousarray(a)).to(torch.device("cuda:0"))
+
+
+@pytest.mark.parametrize("bits", [32, 64])
+@pytest.mark.parametrize("vbits", [32, 64])
+def test_second_level_entry_equals_fusedmm_csr(bits, vbits):
+    """sgfusedMM_csr('g'|'m'|'s'|'t', ...) called through its own symbol gives the
+    bits of fusedMM_csr with the matching op tuple, for beta 0 and 1, host and
+    device operands; an unknown letter prints and leaves C alone (kernels.c:627-629)."""
+    import torch
+    np_v = np.float32 if vbits == 32 else np.float64
+    it, ct = (np.int32, C.c_int32) if bits == 32 else (np.int64, C.c_int64)
+    cv = C.c_float if vbits == 32 else C.c_double
+    lib = fa.load(bits, vbits)
+    gf = lib.sgfusedMM_csr if vbits == 32 else lib.dgfusedMM_csr
+    g = graphs.ragged(bits, hub_deg=900)
+    k = 64
+    X = graphs.features(g["rows"], k, 1, -0.5, 0.5, 1).astype(np_v)
+    Y = graphs.features(g["cols"], k, 1, -0.5, 0.5, 2).astype(np_v)
+    Z0 = graphs.features(g["rows"], k, 1, -1, 1, 3).astype(np_v)
+    val = g["val"].astype(np_v)
+    d = dict(val=_dev(val), indx=_dev(g["indx"]), pb=_dev(g["pntrb"]), pe=_dev(g["pntre"]), X=_dev(X), Y=_dev(Y))
+
+    def second_level(letter, beta, where):
+        if where == "host":
+            Z = Z0.copy()
+            ops = [val, g["indx"], g["pntrb"], g["pntre"], X, Y, Z]
+            addr = [o.ctypes.data for o in ops]
+        else:
+            Zd = _dev(Z0)
+            ops = [d["val"], d["indx"], d["pb"], d["pe"], d["X"], d["Y"], Zd]
+            addr = [o.data_ptr() for o in ops]
+        gf(C.c_char(letter.encode()), ct(g["rows"]), ct(g["cols"]), ct(k), cv(1.0), ct(g["nnz"]), ct(g["rows"]),
+           ct(g["cols"]), addr[0], addr[1], addr[2], addr[3], addr[4], ct(k), addr[5], ct(k), cv(beta), addr[6], ct(k))
+        if where == "host":
+            return Z
+        torch.cuda.synchronize()
+        return Zd.cpu().numpy()
+
+    for letter, kind in (("g", None), ("m", None), ("s", "sigmoid"), ("t", "tdist")):
+        gpu_api.set_kind(SOP_NAMES[kind] if kind else 0, bits, vbits)
+        for beta in (0.0, 1.0):
+            for where in ("device", "host"):
+                print("case", letter, beta, where, bits, vbits, flush=True)
+                rc, want = gpu_api.run(MSG[letter], g, X, Y, Z0, beta=beta, bits=bits, where=where, vbits=vbits)
+                assert rc == 0
+                got = second_level(letter, beta, where)
+                np.testing.assert_array_equal(got.view(np.uint8), want.view(np.uint8))
+                assert not np.array_equal(got, Z0)
+    for where in ("device", "host"):
+        got = second_level("q", 0.0, where)                  # "unknown kernel type!" on stderr, nothing else
+        np.testing.assert_array_equal(got.view(np.uint8), Z0.view(np.uint8))
+
+
+@pytest.mark.parametrize("vbits", [32, 64])
+def test_device_sigmoid_table_equals_the_reference_table(vbits):
+    """The table the kernels index, read back through the kernels themselves:
+    2048 one-edge rows, Y = 1, X[i] = centre of bin i in column 0, sigmoid tuple
+    => Z[i, 0] = 1 - table[i].  Compared bit for bit with the table of the real
+    reference's tester (test/fusedMMtime.cpp:594-604, stored in golden/sop.npz)."""
+    np_v = np.float32 if vbits == 32 else np.float64
+    d = np.load(__import__("os").path.join(GOLD, "sop.npz"))
+    table = d["table" if vbits == 32 else "table_d"]
+    assert table.dtype == np_v and table.size == 2048
+    n, k = 2048, 4
+    it = np.int32
+    g = {"rows": n, "cols": 1, "nnz": n, "val": np.ones(n, np.float32), "indx": np.zeros(n, it),
+         "pntrb": np.arange(n, dtype=it), "pntre": np.arange(1, n + 1, dtype=it)}
+    X = np.zeros((n, k), np_v)
+    X[:, 0] = ((np.arange(n) + 0.5) * 10.0 / 2048 - 5.0).astype(np_v)     # exact in binary: (2i+1) * 5/2048 - 5
+    Y = np.ones((1, k), np_v)
+    gpu_api.set_kind(SOP_NAMES["sigmoid"], 32, vbits)
+    for where in ("device", "host"):
+        rc, Z = gpu_api.run(MSG["s"], g, X, Y, np.zeros((n, k), np_v), bits=32, where=where, vbits=vbits)
+        assert rc == 0
+        want = (np_v(1.0) - table).astype(np_v)
+        np.testing.assert_array_equal(np.ascontiguousarray(Z[:, 0]).view(np.uint8), want.view(np.uint8))
+        np.testing.assert_array_equal(np.ascontiguousarray(Z[:, 3]).view(np.uint8), want.view(np.uint8))
+    # and through the entry point whose table lives in the static array
+    import torch
+    dv = [_dev(g["val"].astype(np_v)), _dev(g["indx"]), _dev(g["pntrb"]), _dev(g["pntre"]), _dev(X), _dev(Y)]
+    Zd = _dev(np.zeros((n, k), np_v))
+    rc = fa.fusedMM_csr(MSG["s"], n, 1, k, 1.0, n, n, 1, dv[0], dv[1], dv[2], dv[3], dv[4], k, dv[5], k, 0.0, Zd, k,
+                        stream=torch.cuda.current_stream().cuda_stream, value_bits=vbits, noalloc=True)
+    assert rc == 0
+    torch.cuda.synchronize()
+    np.testing.assert_array_equal(np.ascontiguousarray(Zd.cpu().numpy()[:, 0]).view(np.uint8), want.view(np.uint8))
+
+
+SOPFN = C.CFUNCTYPE(C.c_int, C.c_float, C.POINTER(C.c_float))
+
+
+def test_operand_check_covers_the_host_function_path():
+    """FUSEDMM_VALIDATE with SOP_UDEF served by the caller's host function: the
+    first pass gathers Y rows by column id and the host walks the row pointers, so
+    bad CSR must be turned away before either happens."""
+    lib = fa.load(32)
+    prev_kind = lib.fusedMM_amd_set_sop_kind(fa.SOP_KIND_HOST)
+    prev = lib.fusedMM_amd_set_validate(1)
+    calls = [0]
+
+    def sop(val, out):
+        calls[0] += 1
+        out[0] = val
+        return 0
+
+    cb = SOPFN(sop)
+    lib.fusedMM_amd_set_sop_callback(C.cast(cb, C.c_void_p))
+    try:
+        g = graphs.tiny_er(50, 120, 2)
+        k = 32
+        X = graphs.features(50, k, 2, -0.5, 0.5, 1)
+        Y = graphs.features(50, k, 2, -0.5, 0.5, 2)
+        Z0 = np.zeros((50, k), np.float32)
+        for where in ("device", "host"):
+            rc, Z = gpu_api.run(MSG["s"], g, X, Y, Z0, where=where)
+            assert rc == 0 and Z.any()
+        seen = calls[0]
+        assert seen == 2 * g["nnz"]
+        bad_col = dict(g)
+        bad_col["indx"] = g["indx"].copy()
+        bad_col["indx"][7] = 50                              # one past the last row of Y
+        bad_end = dict(g)
+        bad_end["pntre"] = g["pntre"].copy()
+        bad_end["pntre"][3] = g["pntrb"][3] - 1
+        bad_start = dict(g)
+        bad_start["pntrb"] = g["pntrb"].copy()
+        bad_start["pntrb"][0] = -4
+        for bad in (bad_col, bad_end, bad_start):
+            for where in ("device", "host"):
+                rc, Z = gpu_api.run(MSG["s"], bad, X, Y, Z0, where=where)
+                assert rc == fa.FAIL and not Z.any()
+        assert calls[0] == seen                              # the user function was never reached
+    finally:
+        lib.fusedMM_amd_set_validate(prev)
+        lib.fusedMM_amd_set_sop_kind(prev_kind)
+        lib.fusedMM_amd_set_sop_callback(None)
+
+
+def test_host_arrays_allocated_exactly_as_far_as_the_reference_reads(oracle):
+    """ld > k with X, Y and Z ending at the last element the reference touches,
+    (rows - 1) * ld + k, each placed at the very end of its own page-aligned
+    mapping so that reading one element further would fault."""
+    import mmap
+    g = graphs.ragged(32, hub_deg=70)
+    k, ldx, ldy, ldz = 48, 52, 64, 56
+
+    def tight(rows, ld, seed, lo, hi):
+        full = graphs.features(rows, ld, 6, lo, hi, seed)
+        used = (rows - 1) * ld + k
+        nbytes = used * 4
+        pages = -(-nbytes // mmap.PAGESIZE)
+        buf = mmap.mmap(-1, (pages + 1) * mmap.PAGESIZE)
+        base = np.frombuffer(buf, np.uint8)
+        # make the page after the data inaccessible
+        libc = C.CDLL(None, use_errno=True)
+        addr = base.ctypes.data
+        assert libc.mprotect(C.c_void_p(addr + pages * mmap.PAGESIZE), C.c_size_t(mmap.PAGESIZE), 0) == 0
+        off = pages * mmap.PAGESIZE - nbytes
+        flat = base[off:off + nbytes].view(np.float32)
+        flat[:] = full.reshape(-1)[:used]
+        return full, flat, buf
+
+    X, Xt, kx = tight(g["rows"], ldx, 1, -0.5, 0.5)
+    Y, Yt, ky = tight(g["cols"], ldy, 2, -0.5, 0.5)
+    Z0, Zt, kz = tight(g["rows"], ldz, 3, -1, 1)
+    gpu_api.set_kind(SOP_NAMES["tdist"], 32)
+    rc = fa.fusedMM_csr(MSG["t"], g["rows"], g["cols"], k, 1.0, g["nnz"], g["rows"], g["cols"], g["val"], g["indx"],
+                        np.ascontiguousarray(g["pntrb"]), np.ascontiguousarray(g["pntre"]), Xt, ldx, Yt, ldy, 1.0, Zt, ldz)
+    assert rc == 0
+    want = Z0.copy()
+    oracle.opt("t", g, X, Y, want, beta=1.0, sop_kind=2, mode=2, V=4, L=16, S=4, k=k)
+    used = (g["rows"] - 1) * ldz + k
+    np.testing.assert_array_equal(np.array(Zt).view(np.uint32), want.reshape(-1)[:used].view(np.uint32))
+
+
+def test_calls_on_different_streams_share_the_queues_safely(oracle):
+    """Every call on a GPU uses that GPU's one set of work queues.  Calls issued
+    back to back on different (non-blocking) streams, with split rows, must each
+    give the single-stream result: the library orders them."""
+    import torch
+    g = graphs.ragged(32, rows=300, cols=4000, hub_deg=30000)
+    k = 128
+    X = graphs.features(g["rows"], k, 3, -0.5, 0.5, 1)
+    Ys = [graphs.features(g["cols"], k, 3 + i, -0.5, 0.5, 2) for i in range(4)]
+    d = dict(val=_dev(g["val"]), indx=_dev(g["indx"]), pb=_dev(g["pntrb"]), pe=_dev(g["pntre"]), X=_dev(X))
+    dY = [_dev(y) for y in Ys]
+    gpu_api.set_kind(SOP_NAMES["sigmoid"], 32)
+
+    def enqueue(Y, Z, stream, noalloc):
+        rc = fa.fusedMM_csr(fa.MSG_SIGMOID, g["rows"], g["cols"], k, 1.0, g["nnz"], g["rows"], g["cols"], d["val"],
+                            d["indx"], d["pb"], d["pe"], d["X"], k, Y, k, 0.0, Z, k, stream=stream, noalloc=noalloc)
+        assert rc == 0
+
+    for noalloc in (False, True):
+        want = []
+        for y in dY:
+            Z = torch.zeros((g["rows"], k), device="cuda:0")
+            enqueue(y, Z, torch.cuda.current_stream().cuda_stream, noalloc)
+            torch.cuda.synchronize()
+            want.append(Z)
+        assert gpu_api.last_split(32)[1] > 0
+        streams = [torch.cuda.Stream() for _ in range(4)]
+        torch.cuda.synchronize()
+        for rep in range(3):
+            got = [torch.full((g["rows"], k), 5.0, device="cuda:0") for _ in range(4)]
+            for i in range(4):
+                enqueue(dY[i], got[i], streams[i].cuda_stream, noalloc)
+            torch.cuda.synchronize()
+            for i in range(4):
+                assert torch.equal(got[i], want[i]), (noalloc, rep, i)
+
+
+def test_nan_dot_product_takes_the_first_table_bin(oracle):
+    """A NaN in X makes the dot NaN; neither saturation test holds for it and the
+    reference converts it to an integer (undefined).  Here the index is clamped to
+    bin 0 on the GPU and in the oracle alike, so the row stays finite."""
+    g = graphs.tiny_er(64, 300, 4)
+    k = 32
+    X = graphs.features(64, k, 5, -0.5, 0.5, 1)
+    Y = graphs.features(64, k, 5, -0.5, 0.5, 2)
+    X[10, 3] = np.nan
+    gpu_api.set_kind(SOP_NAMES["sigmoid"], 32)
+    rc, Z = gpu_api.run(MSG["s"], g, X, Y, np.zeros((64, k), np.float32))
+    assert rc == 0
+    want = np.zeros((64, k), np.float32)
+    oracle.opt("s", g, X, Y, want, sop_kind=1, mode=2, V=4, L=8, S=8)
+    np.testing.assert_array_equal(Z.view(np.uint32), want.view(np.uint32))
+    assert np.isfinite(Z).all() and g["pntre"][10] > g["pntrb"][10]
+    t0 = oracle.table()[0]
+    cols = g["indx"][g["pntrb"][10]:g["pntre"][10]]
+    np.testing.assert_allclose(Z[10], ((np.float32(1) - t0) * Y[cols].astype(np.float64)).sum(0), rtol=1e-5, atol=1e-6)
