@@ -12,6 +12,8 @@
 #include <stdlib.h>
 #include <string.h>
 
+#include <chrono>
+#include <condition_variable>
 #include <mutex>
 #include <thread>
 #include <vector>
@@ -86,16 +88,23 @@ struct DeviceState {
    Counters *ctr = nullptr;
    Buffer heavy, segs, partial, queued;
    Buffer stage[8];           // host-pointer mode: pntrb, pntre, indx, val, x, y, z, spare
+   // host-pointer mode: two pinned buffers each way, copies are pipelined through them
+   void *pin[4] = {nullptr, nullptr, nullptr, nullptr};
+   hipEvent_t pin_ev[4];
+   bool pin_busy[4] = {false, false, false, false};
+   // opt-in device mirrors of read-only host operands, keyed by host address and size
+   struct Mirror { const void *host; size_t bytes; void *dev; unsigned long long last_use; };
+   std::vector<Mirror> mirrors;
    // the static array of this device (address from hipGetSymbolAddress), once set up
    unsigned char *scratch = nullptr;
-   // Calls that share a set of queues must not overlap: each call records order_ev
-   // behind its last kernel, and a call on another stream first waits for it.
+   // Calls that share a set of queues must not overlap: a call on another stream than
+   // the previous one first waits for order_ev, recorded on that earlier stream.
    hipEvent_t order_ev[2];
    hipStream_t last_stream[2] = {nullptr, nullptr};
    bool pending[2] = {false, false};
    Counters *last_ctr = nullptr;   // counters of the most recent call (fusedMM_amd_last_split)
    // timing
-   hipEvent_t ev[kTimingSlots][4];
+   hipEvent_t ev[kTimingSlots][4];   // around the three kernels of a call
    bool ev_made = false;
 };
 
@@ -108,9 +117,14 @@ struct Globals {
    int seg_len = 0;
    int blocks_per_cu = 0;
    int validate = 0;
+   int cache = 0;             // 1: keep device mirrors of read-only host operands between calls
+   unsigned long long cache_clock = 0;
+   double phase_ms[3] = {0, 0, 0};   // upload, kernels, download of the last host-pointer call
+   bool phase_valid = false;
    fusedMM_amd_sop_fn sop_fn = nullptr;
-   bool timing = false;
-   int timing_calls = 0;
+   int timing = 0;            // 0: off; n: HIP events around the kernels of every n-th call
+   int timing_seen = 0;       // calls since timing was switched on
+   int timing_calls = 0;      // calls recorded
    int timing_dev = 0;
    DeviceState dev[kMaxDevices];
 };
@@ -137,6 +151,7 @@ void read_env_once()
    if (const char *e = getenv("FUSEDMM_SOP_KIND")) g.sop_kind = sop_kind_from_name(e);
    if (const char *e = getenv("FUSEDMM_BLOCKS_PER_CU")) g.blocks_per_cu = atoi(e);
    if (const char *e = getenv("FUSEDMM_VALIDATE")) g.validate = atoi(e);
+   if (const char *e = getenv("FUSEDMM_CACHE")) g.cache = atoi(e) ? 1 : 0;
    if (const char *e = getenv("FUSEDMM_SPLIT"))   // "heavy_deg,seg_len", as fusedMM_amd_set_split
    {
       long long h = 0;
@@ -230,7 +245,11 @@ int device_state(DeviceState **out)
 constexpr size_t align256(size_t v) { return (v + 255u) & ~(size_t)255u; }
 constexpr size_t kScratchTableOff = 0;
 constexpr size_t kScratchCtrOff = align256(kSigmoidTableSize * sizeof(val_t));
-constexpr size_t kScratchQueuesOff = kScratchCtrOff + align256(sizeof(Counters));
+constexpr size_t kScratchBitmapOff = kScratchCtrOff + align256(sizeof(Counters));
+// The queued-row bits stay zero between calls only if nothing else is ever written
+// where they live: a fixed region, one bit per row for the largest m accepted.
+constexpr int64_t kScratchMaxRows = (int64_t)1 << 25;
+constexpr size_t kScratchQueuesOff = kScratchBitmapOff + (size_t)(kScratchMaxRows / 8);
 
 // Once per device, with that device current: find this device's copy of the
 // array, put the sigmoid table at its head and zero the counters.
@@ -243,7 +262,7 @@ int scratch_setup(DeviceState &d)
    val_t host_tab[kSigmoidTableSize];
    build_sigmoid_table(host_tab);
    FMM_HIP(hipMemcpy(base + kScratchTableOff, host_tab, sizeof(host_tab), hipMemcpyHostToDevice));
-   FMM_HIP(hipMemset(base + kScratchCtrOff, 0, sizeof(Counters)));
+   FMM_HIP(hipMemset(base + kScratchCtrOff, 0, kScratchQueuesOff - kScratchCtrOff));   // counters and queued-row bits
    d.scratch = base;
    return FUSEDMM_SUCCESS_RETURN;
 }
@@ -392,6 +411,12 @@ int make_plan(int32_t imsg, int opt_enabled, Plan *pl)
    if (opt_enabled && vop == VOP_SUBR && rop == ROP_NORMR && sop == SOP_UDEF && vsc == VSC_MUL && aop == AOP_ADD)
       pl->op = OP_DIST;
    pl->opt_rule = (pl->op != OP_GENERIC);
+   if (opt_enabled == 2 && pl->op == OP_GENERIC)
+   {
+      // the reference built with MUST_OPT_FUSEDMM (fusedMM.c:599-604)
+      FMM_LOG("NO opt implementation for this message! Run the general FusedMM by not requiring the optimised kernels");
+      return FUSEDMM_NO_OPT_IMPL;
+   }
    pl->reads_x = (pl->op == OP_DOT || pl->op == OP_DIST) ||
                  (pl->op == OP_GENERIC && (vop != VOP_COPY_RHS || rop == ROP_DOT || rop == ROP_ADD_LHS || rop == ROP_NORML));
    // the general pipeline seeds the scalar with val[j]; it matters only when no ROP overwrites it
@@ -413,6 +438,26 @@ struct Args {
 int run_on_device(const Args &a, const Plan &pl, int sop_kind, hipStream_t stream, int queues = kQueuesGrown);
 int validate_host_pointers(const Args &h);
 int validate_operands(const Args &a, hipStream_t stream, int queues = kQueuesGrown);
+
+// Make `stream` wait for the work of the previous call that used this set of
+// queues, when that call went to another stream.  The event is recorded only now,
+// on that earlier stream (it then covers the earlier call and whatever the caller
+// enqueued there since): a record after every call would sit between consecutive
+// calls of the common one-stream case and keep them from running back to back.
+int order_after_previous(DeviceState &d, int queues, hipStream_t stream)
+{
+   if (!d.pending[queues] || d.last_stream[queues] == stream) return FUSEDMM_SUCCESS_RETURN;
+   hipError_t e = hipEventRecord(d.order_ev[queues], d.last_stream[queues]);
+   if (e == hipSuccess) e = hipStreamWaitEvent(stream, d.order_ev[queues], 0);
+   if (e != hipSuccess)
+   {
+      // the earlier stream is gone (destroyed by the caller; its work still completes)
+      (void)hipGetLastError();
+      FMM_HIP(hipDeviceSynchronize());
+   }
+   d.pending[queues] = false;
+   return FUSEDMM_SUCCESS_RETURN;
+}
 
 // Is `stream` being recorded into a HIP graph?  The legacy default stream cannot be.
 int stream_capturing(hipStream_t stream, bool *capturing)
@@ -506,10 +551,10 @@ int run_slab(const Args &a, const Plan &pl, int sop_kind, hipStream_t stream, in
    {
       // same capacities as the allocating entry points (so the same rows are split and
       // the results are the same bits), laid out behind the fixed head of the array
-      const size_t o_queued = kScratchQueuesOff, o_heavy = o_queued + align256(b_queued),
+      const size_t o_queued = kScratchBitmapOff, o_heavy = kScratchQueuesOff,
                    o_segs = o_heavy + align256(b_heavy), o_partial = o_segs + align256(b_segs),
                    end = o_partial + align256(b_partial);
-      if (end > (size_t)FUSEDMM_AMD_SCRATCH_BYTES)
+      if (a.m > kScratchMaxRows || end > (size_t)FUSEDMM_AMD_SCRATCH_BYTES)
       {
          FMM_LOG("fusedMM_csr_stream_noalloc: m=%lld, nnz=%lld, k=%lld need %zu bytes of work queues; the static "
                  "array holds %zu (use fusedMM_csr_stream for this size)",
@@ -529,7 +574,13 @@ int run_slab(const Args &a, const Plan &pl, int sop_kind, hipStream_t stream, in
       st = grow(d->heavy, b_heavy, capturing); if (st) return st;
       st = grow(d->segs, b_segs, capturing); if (st) return st;
       st = grow(d->partial, b_partial, capturing); if (st) return st;
-      st = grow(d->queued, b_queued, capturing); if (st) return st;
+      {
+         // the queued-row bits are zero between calls (the fused kernel's last wavefront
+         // clears what the call set), so a new buffer starts out zero and stays that way
+         const void *before = d->queued.ptr;
+         st = grow(d->queued, b_queued, capturing); if (st) return st;
+         if (d->queued.ptr != before) FMM_HIP(hipMemsetAsync(d->queued.ptr, 0, d->queued.bytes, stream));
+      }
       p.sigmoid_table = d->sigmoid_table;
       p.ctr = d->ctr;
       p.heavy = (HeavyRow *)d->heavy.ptr;
@@ -542,17 +593,13 @@ int run_slab(const Args &a, const Plan &pl, int sop_kind, hipStream_t stream, in
    d->last_ctr = p.ctr;
 
    // Calls that share these queues must run one after the other.  On one stream
-   // they do; a call on another stream first waits for the previous call's last
-   // kernel.  (Not while capturing: an event recorded into a graph cannot be
+   // they do; a call on another stream first waits for what the previous call's
+   // stream holds.  (Not while capturing: an event recorded into a graph cannot be
    // waited on from outside it; the graph's launches are ordered by their stream.)
-   if (!capturing && d->pending[queues] && d->last_stream[queues] != stream)
-      FMM_HIP(hipStreamWaitEvent(stream, d->order_ev[queues], 0));
-
+   if (!capturing)
    {
-      int64_t rb = (queued_words + kBlockThreads - 1) / kBlockThreads;
-      if (rb > (int64_t)d->num_cu * 4) rb = (int64_t)d->num_cu * 4;
-      if (rb < 1) rb = 1;
-      hipLaunchKernelGGL(reset_kernel, dim3((unsigned int)rb), dim3(kBlockThreads), 0, stream, p.ctr, p.queued, queued_words);
+      st = order_after_previous(*d, queues, stream);
+      if (st) return st;
    }
 
    Launch l;
@@ -561,7 +608,8 @@ int run_slab(const Args &a, const Plan &pl, int sop_kind, hipStream_t stream, in
    l.nnz_hint = nnz_hint;
    l.stream = stream;
    l.ev = nullptr;
-   if (g.timing && g.timing_calls < kTimingSlots && queues == kQueuesGrown && !capturing)
+   if (g.timing > 0 && queues == kQueuesGrown && !capturing && (g.timing_seen++ % g.timing) == 0 &&
+       g.timing_calls < kTimingSlots)
    {
       if (!d->ev_made)
       {
@@ -591,7 +639,6 @@ int run_slab(const Args &a, const Plan &pl, int sop_kind, hipStream_t stream, in
    if (st) return st;
    if (!capturing)
    {
-      FMM_HIP(hipEventRecord(d->order_ev[queues], stream));
       d->pending[queues] = true;
       d->last_stream[queues] = stream;
    }
@@ -632,6 +679,170 @@ int operand_residence(const Args &a)
    return dev ? 1 : 0;
 }
 
+// ---- host-pointer mode: pinned staging ------------------------------------------------
+// The caller's arrays are ordinary pageable memory.  They move through two pinned
+// buffers each way, 16 MiB at a time: a few threads copy chunk i+1 between the
+// caller's array and a pinned buffer while the DMA engine moves chunk i.
+constexpr size_t kPinChunk = (size_t)16 << 20;
+constexpr size_t kPinMinBytes = (size_t)1 << 20;   // smaller copies go straight through hipMemcpyAsync
+
+class CopyPool {
+ public:
+   void copy(void *dst, const void *src, size_t bytes)
+   {
+      if (bytes < ((size_t)1 << 20) || !start()) { memcpy(dst, src, bytes); return; }
+      std::unique_lock<std::mutex> lk(m_);
+      dst_ = (char *)dst; src_ = (const char *)src; bytes_ = bytes;
+      remaining_ = (int)th_.size();
+      generation_++;
+      cv_.notify_all();
+      done_.wait(lk, [&] { return remaining_ == 0; });
+   }
+   ~CopyPool()
+   {
+      {
+         std::lock_guard<std::mutex> lk(m_);
+         stop_ = true;
+         generation_++;
+      }
+      cv_.notify_all();
+      for (auto &t : th_) t.join();
+   }
+
+ private:
+   bool start()
+   {
+      if (!th_.empty()) return true;
+      unsigned int n = std::thread::hardware_concurrency();
+      n = n < 2 ? 0 : (n > 8 ? 8 : n);
+      for (unsigned int i = 0; i < n; i++) th_.emplace_back([this, i, n] { work(i, n); });
+      return n > 0;
+   }
+   void work(unsigned int i, unsigned int n)
+   {
+      int seen = 0;
+      for (;;)
+      {
+         std::unique_lock<std::mutex> lk(m_);
+         cv_.wait(lk, [&] { return generation_ != seen; });
+         seen = generation_;
+         if (stop_) return;
+         char *d = dst_; const char *s = src_; const size_t b = bytes_;
+         lk.unlock();
+         const size_t lo = b / n * i, hi = (i + 1 == n) ? b : b / n * (i + 1);
+         memcpy(d + lo, s + lo, hi - lo);
+         lk.lock();
+         if (--remaining_ == 0) done_.notify_one();
+      }
+   }
+   std::vector<std::thread> th_;
+   std::mutex m_;
+   std::condition_variable cv_, done_;
+   char *dst_ = nullptr; const char *src_ = nullptr; size_t bytes_ = 0;
+   int generation_ = 0, remaining_ = 0;
+   bool stop_ = false;
+};
+CopyPool copy_pool;
+
+int pinned_buffers(DeviceState &d)
+{
+   if (d.pin[0]) return FUSEDMM_SUCCESS_RETURN;
+   for (int i = 0; i < 4; i++)
+   {
+      FMM_HIP(hipHostMalloc(&d.pin[i], kPinChunk, hipHostMallocDefault));
+      FMM_HIP(hipEventCreateWithFlags(&d.pin_ev[i], hipEventDisableTiming));
+      d.pin_busy[i] = false;
+   }
+   return FUSEDMM_SUCCESS_RETURN;
+}
+
+// host -> device, enqueued on `s`; returns when the host array has been read
+int upload(DeviceState &d, void *dev, const void *host, size_t bytes, hipStream_t s)
+{
+   if (bytes == 0) return FUSEDMM_SUCCESS_RETURN;
+   if (bytes < kPinMinBytes) { FMM_HIP(hipMemcpyAsync(dev, host, bytes, hipMemcpyHostToDevice, s)); return FUSEDMM_SUCCESS_RETURN; }
+   int st = pinned_buffers(d);
+   if (st) return st;
+   int b = 0;
+   for (size_t off = 0; off < bytes; off += kPinChunk, b ^= 1)
+   {
+      const size_t n = bytes - off < kPinChunk ? bytes - off : kPinChunk;
+      if (d.pin_busy[b]) FMM_HIP(hipEventSynchronize(d.pin_ev[b]));   // its previous DMA has drained
+      copy_pool.copy(d.pin[b], (const char *)host + off, n);
+      FMM_HIP(hipMemcpyAsync((char *)dev + off, d.pin[b], n, hipMemcpyHostToDevice, s));
+      FMM_HIP(hipEventRecord(d.pin_ev[b], s));
+      d.pin_busy[b] = true;
+   }
+   return FUSEDMM_SUCCESS_RETURN;
+}
+
+// device -> host through the other two pinned buffers; returns when `host` holds the data
+int download(DeviceState &d, void *host, const void *dev, size_t bytes, hipStream_t s)
+{
+   if (bytes == 0) return FUSEDMM_SUCCESS_RETURN;
+   if (bytes < kPinMinBytes)
+   {
+      FMM_HIP(hipMemcpyAsync(host, dev, bytes, hipMemcpyDeviceToHost, s));
+      return hip_status(hipStreamSynchronize(s), "hipStreamSynchronize");
+   }
+   int st = pinned_buffers(d);
+   if (st) return st;
+   size_t prev_off = 0, prev_n = 0;
+   int b = 2, prev_b = -1;
+   for (size_t off = 0; off < bytes; off += kPinChunk)
+   {
+      const size_t n = bytes - off < kPinChunk ? bytes - off : kPinChunk;
+      FMM_HIP(hipMemcpyAsync(d.pin[b], (const char *)dev + off, n, hipMemcpyDeviceToHost, s));
+      FMM_HIP(hipEventRecord(d.pin_ev[b], s));
+      if (prev_b >= 0)
+      {
+         FMM_HIP(hipEventSynchronize(d.pin_ev[prev_b]));
+         copy_pool.copy((char *)host + prev_off, d.pin[prev_b], prev_n);
+      }
+      prev_b = b; prev_off = off; prev_n = n;
+      b = (b == 2) ? 3 : 2;
+   }
+   FMM_HIP(hipEventSynchronize(d.pin_ev[prev_b]));
+   copy_pool.copy((char *)host + prev_off, d.pin[prev_b], prev_n);
+   d.pin_busy[2] = d.pin_busy[3] = false;
+   return FUSEDMM_SUCCESS_RETURN;
+}
+
+// Device copy of a read-only host operand.  With the mirror cache off (the
+// default) it is uploaded into the staging buffer `stage` on every call, as
+// the caller may have changed it.  With the cache on, a mirror keyed by host
+// address and size is kept and reused until fusedMM_amd_invalidate().
+int device_copy(DeviceState &d, Buffer &stage, const void *host, size_t bytes, size_t copy_bytes, hipStream_t s, const void **out)
+{
+   if (!g.cache)
+   {
+      int st = grow(stage, bytes);
+      if (st) return st;
+      *out = stage.ptr;
+      return upload(d, stage.ptr, host, copy_bytes, s);
+   }
+   for (auto &mi : d.mirrors)
+      if (mi.host == host && mi.bytes == copy_bytes)
+      {
+         mi.last_use = ++g.cache_clock;
+         *out = mi.dev;
+         return FUSEDMM_SUCCESS_RETURN;
+      }
+   if (d.mirrors.size() >= 32)   // drop the mirror used longest ago
+   {
+      size_t victim = 0;
+      for (size_t i = 1; i < d.mirrors.size(); i++)
+         if (d.mirrors[i].last_use < d.mirrors[victim].last_use) victim = i;
+      (void)hipFree(d.mirrors[victim].dev);
+      d.mirrors.erase(d.mirrors.begin() + (long)victim);
+   }
+   void *dev = nullptr;
+   FMM_HIP(hipMalloc(&dev, bytes > 0 ? bytes : 16));
+   d.mirrors.push_back(DeviceState::Mirror{host, copy_bytes, dev, ++g.cache_clock});
+   *out = dev;
+   return upload(d, dev, host, copy_bytes, s);
+}
+
 // Host-pointer mode: copy the operands to the GPU.  On return `a` holds device
 // addresses and `slots` is one past the last edge slot any processed row uses.
 int stage_up(const Args &h, const Plan &pl, Args *a, int64_t *slots_out)
@@ -666,33 +877,34 @@ int stage_up(const Args &h, const Plan &pl, Args *a, int64_t *slots_out)
    const size_t b_x = (size_t)h.m * (size_t)h.ldx * kValBytes;
    const size_t b_y = (size_t)h.n * (size_t)h.ldy * kValBytes;
    const size_t b_z = (size_t)h.m * (size_t)h.ldz * kValBytes;
-   st = grow(d->stage[0], b_ptr); if (st) return st;
-   st = grow(d->stage[1], b_ptr); if (st) return st;
-   st = grow(d->stage[2], b_idx); if (st) return st;
-   if (need_val) { st = grow(d->stage[3], b_val); if (st) return st; }
-   if (pl.reads_x) { st = grow(d->stage[4], b_x); if (st) return st; }
-   st = grow(d->stage[5], b_y); if (st) return st;
-   st = grow(d->stage[6], b_z); if (st) return st;
-
-   hipStream_t s = 0;
-   FMM_HIP(hipMemcpyAsync(d->stage[0].ptr, h.pntrb, b_ptr, hipMemcpyHostToDevice, s));
-   FMM_HIP(hipMemcpyAsync(d->stage[1].ptr, h.pntre, b_ptr, hipMemcpyHostToDevice, s));
-   if (slots > 0) FMM_HIP(hipMemcpyAsync(d->stage[2].ptr, h.indx, (size_t)slots * sizeof(idx_t), hipMemcpyHostToDevice, s));
-   if (need_val && slots > 0) FMM_HIP(hipMemcpyAsync(d->stage[3].ptr, h.val, (size_t)slots * kValBytes, hipMemcpyHostToDevice, s));
    // the caller's arrays need not extend past the last element the reference reads:
    // (rows - 1) * ld + k elements, not rows * ld
-   if (pl.reads_x) FMM_HIP(hipMemcpyAsync(d->stage[4].ptr, h.x, b_x - (size_t)(h.ldx - h.k) * kValBytes, hipMemcpyHostToDevice, s));
-   FMM_HIP(hipMemcpyAsync(d->stage[5].ptr, h.y, b_y - (size_t)(h.ldy - h.k) * kValBytes, hipMemcpyHostToDevice, s));
+   hipStream_t s = 0;
+   const void *dp[6] = {nullptr, nullptr, nullptr, nullptr, nullptr, nullptr};
+   st = device_copy(*d, d->stage[0], h.pntrb, b_ptr, b_ptr, s, &dp[0]); if (st) return st;
+   st = device_copy(*d, d->stage[1], h.pntre, b_ptr, b_ptr, s, &dp[1]); if (st) return st;
+   st = device_copy(*d, d->stage[2], h.indx, b_idx, (size_t)slots * sizeof(idx_t), s, &dp[2]); if (st) return st;
+   if (need_val) { st = device_copy(*d, d->stage[3], h.val, b_val, (size_t)slots * kValBytes, s, &dp[3]); if (st) return st; }
+   st = device_copy(*d, d->stage[5], h.y, b_y, b_y - (size_t)(h.ldy - h.k) * kValBytes, s, &dp[5]); if (st) return st;
+   if (pl.reads_x)
+   {
+      if ((const void *)h.x == (const void *)h.y && h.ldx == h.ldy && b_x <= b_y) dp[4] = dp[5];   // A = B: one copy serves both
+      else { st = device_copy(*d, d->stage[4], h.x, b_x, b_x - (size_t)(h.ldx - h.k) * kValBytes, s, &dp[4]); if (st) return st; }
+   }
+   st = grow(d->stage[6], b_z); if (st) return st;
    const bool overwrite = pl.opt_rule && h.beta == 0.0f;
    if (!overwrite)   // one contiguous copy, padding columns included (they are never written back)
-      FMM_HIP(hipMemcpyAsync(d->stage[6].ptr, h.z, b_z - (size_t)(h.ldz - h.k) * kValBytes, hipMemcpyHostToDevice, s));
+   {
+      st = upload(*d, d->stage[6].ptr, h.z, b_z - (size_t)(h.ldz - h.k) * kValBytes, s);
+      if (st) return st;
+   }
    *a = h;
-   a->pntrb = (const idx_t *)d->stage[0].ptr;
-   a->pntre = (const idx_t *)d->stage[1].ptr;
-   a->indx = (const idx_t *)d->stage[2].ptr;
-   a->val = need_val ? (const val_t *)d->stage[3].ptr : nullptr;
-   a->x = pl.reads_x ? (const val_t *)d->stage[4].ptr : nullptr;
-   a->y = (const val_t *)d->stage[5].ptr;
+   a->pntrb = (const idx_t *)dp[0];
+   a->pntre = (const idx_t *)dp[1];
+   a->indx = (const idx_t *)dp[2];
+   a->val = need_val ? (const val_t *)dp[3] : nullptr;
+   a->x = pl.reads_x ? (const val_t *)dp[4] : nullptr;
+   a->y = (const val_t *)dp[5];
    a->z = (val_t *)d->stage[6].ptr;
    if (a->nnz <= 0 || a->nnz > slots) a->nnz = slots;
    *slots_out = slots;
@@ -706,16 +918,14 @@ int stage_up(const Args &h, const Plan &pl, Args *a, int64_t *slots_out)
 // slower than either).
 int stage_down(const Args &h, const Args &a)
 {
+   DeviceState *d = nullptr;
+   int st = device_state(&d);
+   if (st) return st;
    const size_t span = ((size_t)h.m * (size_t)h.ldz - (size_t)(h.ldz - h.k)) * kValBytes;
-   if (h.ldz == h.k)
-   {
-      FMM_HIP(hipMemcpyAsync(h.z, a.z, span, hipMemcpyDeviceToHost, 0));
-      FMM_HIP(hipStreamSynchronize(0));
-      return FUSEDMM_SUCCESS_RETURN;
-   }
+   if (h.ldz == h.k) return download(*d, h.z, a.z, span, 0);
    std::vector<val_t> tmp(span / kValBytes);
-   FMM_HIP(hipMemcpyAsync(tmp.data(), a.z, span, hipMemcpyDeviceToHost, 0));
-   FMM_HIP(hipStreamSynchronize(0));
+   st = download(*d, tmp.data(), a.z, span, 0);
+   if (st) return st;
    for (int64_t i = 0; i < h.m; i++)
       memcpy(h.z + i * h.ldz, tmp.data() + i * h.ldz, (size_t)h.k * kValBytes);
    return FUSEDMM_SUCCESS_RETURN;
@@ -724,10 +934,16 @@ int stage_down(const Args &h, const Args &a)
 int run_staged(const Args &h, const Plan &pl, int sop_kind)
 {
    if (h.m <= 0 || h.k < 1) return FUSEDMM_SUCCESS_RETURN;
+   typedef std::chrono::steady_clock clk;
+   auto ms = [](clk::time_point a, clk::time_point b) { return std::chrono::duration<double, std::milli>(b - a).count(); };
+   g.phase_valid = false;
+   const clk::time_point t0 = clk::now();
    Args a;
    int64_t slots = 0;
    int st = stage_up(h, pl, &a, &slots);
    if (st) return st;
+   FMM_HIP(hipStreamSynchronize(0));
+   const clk::time_point t1 = clk::now();
    if (g.validate)
    {
       st = validate_operands(a, 0);
@@ -735,7 +951,14 @@ int run_staged(const Args &h, const Plan &pl, int sop_kind)
    }
    st = run_on_device(a, pl, sop_kind, 0);
    if (st) return st;
-   return stage_down(h, a);
+   FMM_HIP(hipStreamSynchronize(0));
+   const clk::time_point t2 = clk::now();
+   st = stage_down(h, a);
+   if (st) return st;
+   const clk::time_point t3 = clk::now();
+   g.phase_ms[0] = ms(t0, t1); g.phase_ms[1] = ms(t1, t2); g.phase_ms[2] = ms(t2, t3);
+   g.phase_valid = true;
+   return FUSEDMM_SUCCESS_RETURN;
 }
 
 // ---- SOP_UDEF evaluated by the caller's host function ---------------------------------------
@@ -803,7 +1026,10 @@ int validate_operands(const Args &a, hipStream_t stream, int queues)
    memset(&p, 0, sizeof(p));
    p.pntrb = a.pntrb; p.pntre = a.pntre; p.indx = a.indx; p.m = a.m;
    // the flag is one of the shared counters: wait for a call still using them on another stream
-   if (d->pending[queues] && d->last_stream[queues] != stream) FMM_HIP(hipStreamWaitEvent(stream, d->order_ev[queues], 0));
+   st = order_after_previous(*d, queues, stream);
+   if (st) return st;
+   d->pending[queues] = true;
+   d->last_stream[queues] = stream;
    unsigned int *flag = &ctr->invalid;
    FMM_HIP(hipMemsetAsync(flag, 0, sizeof(unsigned int), stream));
    int64_t blocks = (a.m + kWavesPerBlock - 1) / kWavesPerBlock;
@@ -1178,8 +1404,44 @@ int fusedMM_amd_set_opt(int enable)
 {
    std::lock_guard<std::mutex> lock(g.mu);
    int prev = g.opt;
-   g.opt = enable ? 1 : 0;
+   g.opt = enable < 0 ? 0 : (enable > 2 ? 2 : enable);
    return prev;
+}
+
+int fusedMM_amd_set_cache(int enable)
+{
+   std::lock_guard<std::mutex> lock(g.mu);
+   read_env_once();
+   int prev = g.cache;
+   g.cache = enable ? 1 : 0;
+   return prev;
+}
+
+void fusedMM_amd_invalidate(void)
+{
+   std::lock_guard<std::mutex> lock(g.mu);
+   int cur = 0;
+   if (hipGetDevice(&cur) != hipSuccess) return;
+   for (int dev = 0; dev < kMaxDevices; dev++)
+   {
+      DeviceState &d = g.dev[dev];
+      if (d.mirrors.empty()) continue;
+      if (hipSetDevice(dev) != hipSuccess) continue;
+      (void)hipDeviceSynchronize();
+      for (auto &mi : d.mirrors) (void)hipFree(mi.dev);
+      d.mirrors.clear();
+   }
+   (void)hipSetDevice(cur);
+}
+
+int fusedMM_amd_last_host_phases(double *upload_ms, double *kernels_ms, double *download_ms)
+{
+   std::lock_guard<std::mutex> lock(g.mu);
+   if (!g.phase_valid) return FUSEDMM_FAIL_RETURN;
+   if (upload_ms) *upload_ms = g.phase_ms[0];
+   if (kernels_ms) *kernels_ms = g.phase_ms[1];
+   if (download_ms) *download_ms = g.phase_ms[2];
+   return FUSEDMM_SUCCESS_RETURN;
 }
 
 int fusedMM_amd_set_validate(int enable)
@@ -1201,7 +1463,8 @@ void fusedMM_amd_set_split(int64_t heavy_deg, int seg_len)
 void fusedMM_amd_timing(int enable)
 {
    std::lock_guard<std::mutex> lock(g.mu);
-   g.timing = enable != 0;
+   g.timing = enable > 0 ? enable : 0;
+   g.timing_seen = 0;
    g.timing_calls = 0;
 }
 
@@ -1254,9 +1517,9 @@ int fusedMM_amd_last_split(unsigned int *heavy_rows, unsigned int *segments, uns
    memset(&c, 0, sizeof(c));
    FMM_HIP(hipDeviceSynchronize());
    if (d->last_ctr) FMM_HIP(hipMemcpy(&c, d->last_ctr, sizeof(c), hipMemcpyDeviceToHost));
-   if (heavy_rows) *heavy_rows = c.n_heavy;
-   if (segments) *segments = c.n_seg;
-   if (overflow) *overflow = c.overflow;
+   if (heavy_rows) *heavy_rows = c.last_heavy;
+   if (segments) *segments = c.last_seg;
+   if (overflow) *overflow = c.last_overflow;
    return FUSEDMM_SUCCESS_RETURN;
 }
 
@@ -1270,6 +1533,31 @@ int fusedMM_amd_copy_probe(void *dst, const void *src, int64_t bytes, void *stre
    hipLaunchKernelGGL(copy_probe_kernel, dim3((unsigned int)(d->num_cu * 8)), dim3(kBlockThreads), 0, (hipStream_t)stream,
                       (float4 *)dst, (const float4 *)src, bytes / 16);
    return hip_status(hipGetLastError(), "copy probe launch");
+}
+
+int fusedMM_amd_read_probe(const void *src, int64_t bytes, int blocks_per_cu, int in_flight, int nontemporal,
+                           void *sink, void *stream)
+{
+   if (!src || !sink || bytes < 16 || (bytes & 15) || !aligned16(src)) return FUSEDMM_FAIL_RETURN;
+   std::lock_guard<std::mutex> lock(g.mu);
+   DeviceState *d = nullptr;
+   int st = device_basics(&d);
+   if (st) return st;
+   if (blocks_per_cu < 1) blocks_per_cu = 8;
+   const dim3 grid((unsigned int)(d->num_cu * blocks_per_cu)), block(kBlockThreads);
+   const probe16_t *s4 = (const probe16_t *)src;
+   unsigned int *out = (unsigned int *)sink;
+   const int64_t n16 = bytes / 16;
+   hipStream_t hs = (hipStream_t)stream;
+#define FMM_PROBE(U_)                                                                                     \
+   if (nontemporal) hipLaunchKernelGGL((read_probe_kernel<U_, true>), grid, block, 0, hs, s4, n16, out);  \
+   else hipLaunchKernelGGL((read_probe_kernel<U_, false>), grid, block, 0, hs, s4, n16, out)
+   if (in_flight >= 16) { FMM_PROBE(16); }
+   else if (in_flight >= 8) { FMM_PROBE(8); }
+   else if (in_flight >= 4) { FMM_PROBE(4); }
+   else { FMM_PROBE(2); }
+#undef FMM_PROBE
+   return hip_status(hipGetLastError(), "read probe launch");
 }
 
 void fusedMM_amd_finalize(void)
@@ -1289,10 +1577,14 @@ void fusedMM_amd_finalize(void)
       Buffer *bufs[] = {&d.heavy, &d.segs, &d.partial, &d.queued};
       for (Buffer *b : bufs) { if (b->ptr) (void)hipFree(b->ptr); *b = Buffer(); }
       for (Buffer &b : d.stage) { if (b.ptr) (void)hipFree(b.ptr); b = Buffer(); }
+      for (auto &mi : d.mirrors) (void)hipFree(mi.dev);
+      d.mirrors.clear();
+      if (d.pin[0])
+         for (int i = 0; i < 4; i++) { (void)hipHostFree(d.pin[i]); (void)hipEventDestroy(d.pin_ev[i]); }
       if (d.ev_made)
          for (int i = 0; i < kTimingSlots; i++)
             for (int e = 0; e < 4; e++) (void)hipEventDestroy(d.ev[i][e]);
-      d = DeviceState();
+      d = DeviceState();   // also forgets the static array's address: its head is cleared again on next use
    }
    (void)hipSetDevice(cur);
 }

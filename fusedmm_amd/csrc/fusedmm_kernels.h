@@ -51,17 +51,28 @@ constexpr int kSigmoidTableSize = 2048;
 constexpr int kBlockThreads = 256;
 constexpr int kWavesPerBlock = kBlockThreads / 64;
 
+// Queue and claim counters of one call.  The queue counters, the row and retire
+// counters are zero between calls: the last workgroup of the fused kernel to
+// finish puts them back (and clears the queued-row bits), so a call needs no
+// reset pass of its own.
 struct Counters {
    unsigned int n_heavy;    // heavy rows queued by the classify kernel
    unsigned int n_seg;      // edge segments queued
    unsigned int overflow;   // heavy rows that did not fit the queue (processed whole in phase B)
+   unsigned int done_groups; // groups of workgroups of the fused kernel that have finished (see retire[])
    unsigned int invalid;    // set by the optional operand check
-   unsigned int pad2[28];         // keep the row counters on their own 128-byte lines
+   unsigned int last_heavy, last_seg, last_overflow;   // n_heavy, n_seg, overflow of the call that finished last
+   unsigned int merge_heavy;      // heavy rows the merge kernel of this call has to fold (n_heavy, capped)
+   unsigned int pad2[23];         // keep the row counters on their own 128-byte lines
    // Row claim counters.  Read-modify-writes on ONE address retire one per
    // ~12 ns on this GPU however many CUs issue them; on distinct 128-byte
    // lines they proceed in parallel.  So the row space is dealt to
    // kRowCounters counters and a wave works its home counter first.
    struct alignas(128) RowCounter { unsigned long long next; } rows[64];
+   // Workgroups of the fused kernel that have finished, counted per group of
+   // workgroups (blockIdx % 64) for the same reason: one shared counter would
+   // make the kernel's end wait ~12 ns per workgroup.
+   struct alignas(128) RetireCounter { unsigned int done; } retire[64];
 };
 constexpr int kRowCounters = 64;
 
@@ -874,6 +885,12 @@ __device__ __forceinline__ void rows_phase(const Params<IdxT> &p, const real_t *
       my_e = p.pntre[row0 + lane];
    }
    if (nc > 0 && lane == 0) claimed = atomicAdd(&p.ctr->rows[cur].next, 1ull);
+   // rows of this claim that have edges, one bit per row: while a row is walked, the
+   // first column ids and the X slice of the next such row are already on their way
+   const unsigned int has_edges = (unsigned int)__ballot(lane < kRowsPerClaim && my_e > my_b);
+   EdgeChunk<IdxT> first;
+   Slice<R> xs_next;
+   int fetched_t = -1;        // row of this claim whose first chunk `first` (and X slice `xs_next`) hold
    for (int t = 0; t < kRowsPerClaim && row0 + t < p.m; t++)
    {
       const int64_t row = row0 + t;
@@ -903,17 +920,23 @@ __device__ __forceinline__ void rows_phase(const Params<IdxT> &p, const real_t *
          }
          continue;
       }
+      if (generic && aop == kAopNoop) continue;   // general semantics with no accumulate stage: Z is left alone
+
       Slice<R> xs, acc;
-      if (reads_x) load_slice<V, L, R, EXACT, true>(xs, p.x + row * p.ldx, sl, p.k);
+      if (fetched_t == t) xs = xs_next;
       else
       {
+         if (reads_x) load_slice<V, L, R, EXACT, true>(xs, p.x + row * p.ldx, sl, p.k);
+         else
+         {
 #pragma unroll
-         for (int r = 0; r < R; r++) xs.v[r] = zero4();
+            for (int r = 0; r < R; r++) xs.v[r] = zero4();
+         }
+         load_chunk<OP, IdxT>(first, p, jb, je, lane);
       }
       if (generic)
       {
          // general semantics: fold the edges into the caller's Z with AOP
-         if (aop == kAopNoop) continue;
          if (sub == 0) load_slice<V, L, R, EXACT>(acc, zrow, sl, p.k);
          else
          {
@@ -928,9 +951,24 @@ __device__ __forceinline__ void rows_phase(const Params<IdxT> &p, const real_t *
          for (int r = 0; r < R; r++) acc.v[r] = zero4();
       }
 
-      EdgeChunk<IdxT> first;
-      load_chunk<OP, IdxT>(first, p, jb, je, lane);
-      walk_edges<V, L, R, EXACT, OP, SOPK, U, IdxT>(acc, xs, p, jb, je, first, (IdxT)0, (IdxT)0, lane, tab);
+      // next row of the claim with edges: its X slice is requested now, its first 64
+      // column ids by the walk below while this row's last chunk is gathered
+      const unsigned int later = (t + 1 < kRowsPerClaim) ? (has_edges >> (t + 1)) : 0u;
+      IdxT nb = 0, ne = 0;
+      fetched_t = -1;
+      if (later)
+      {
+         fetched_t = t + 1 + __builtin_ctz(later);
+         nb = lane_value<IdxT>(my_b, fetched_t);
+         ne = lane_value<IdxT>(my_e, fetched_t);
+         if (reads_x) load_slice<V, L, R, EXACT, true>(xs_next, p.x + (row0 + fetched_t) * p.ldx, sl, p.k);
+         else
+         {
+#pragma unroll
+            for (int r = 0; r < R; r++) xs_next.v[r] = zero4();
+         }
+      }
+      walk_edges<V, L, R, EXACT, OP, SOPK, U, IdxT>(acc, xs, p, jb, je, first, nb, ne, lane, tab);
       merge_subwaves<L, R, OP>(acc, p.imessage);
 
       if (sub == 0)
@@ -948,6 +986,52 @@ __device__ __forceinline__ void rows_phase(const Params<IdxT> &p, const real_t *
    }
 }
 
+// Every wavefront ends here.  The last workgroup to finish, when nobody reads the
+// queues any more, puts them back to their resting state for the next call: the
+// bits of the queued rows cleared, the counters zero (their values kept in
+// last_*, and the number of rows to fold handed to the merge kernel in
+// merge_heavy).  "Last" is found in two steps, workgroups counting into one of 64
+// group counters and complete groups into one more, so that no counter sees more
+// than a few dozen read-modify-writes.
+template <typename IdxT>
+__device__ __forceinline__ void retire_wave(const Params<IdxT> &p)
+{
+   const int lane = threadIdx.x & 63;
+   __syncthreads();                       // the whole workgroup is done with the queues
+   if (threadIdx.x >= 64) return;
+   Counters *c = p.ctr;
+   const unsigned int groups = gridDim.x < 64u ? gridDim.x : 64u;
+   const unsigned int grp = blockIdx.x & 63u;
+   const unsigned int in_group = (gridDim.x - grp + 63u) / 64u;   // workgroups b with b % 64 == grp
+   unsigned int before = 0u;
+   if (lane == 0) before = __hip_atomic_fetch_add(&c->retire[grp].done, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+   before = (unsigned int)__builtin_amdgcn_readfirstlane((int)before);
+   if (before + 1u != in_group) return;
+   if (lane == 0) before = __hip_atomic_fetch_add(&c->done_groups, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+   before = (unsigned int)__builtin_amdgcn_readfirstlane((int)before);
+   if (before + 1u != groups) return;
+   __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
+   const unsigned int queued_heavy = c->n_heavy < p.cap_heavy ? c->n_heavy : p.cap_heavy;
+   for (unsigned int h = lane; h < queued_heavy; h += 64)
+   {
+      const HeavyRow hr = p.heavy[h];
+      if (hr.n_seg) p.queued[hr.row >> 5] = 0u;   // every bit of the word belongs to a row on this list
+   }
+   c->rows[lane].next = 0ull;
+   c->retire[lane].done = 0u;
+   if (lane == 0)
+   {
+      c->last_heavy = c->n_heavy;
+      c->last_seg = c->n_seg;
+      c->last_overflow = c->overflow;
+      c->merge_heavy = queued_heavy;
+      c->n_heavy = 0u;
+      c->n_seg = 0u;
+      c->overflow = 0u;
+      c->done_groups = 0u;
+   }
+}
+
 // ---- kernel 2: the fused SDDMM+SpMM kernel ------------------------------------------
 // Long work first: every wave takes its share of the queued segments of heavy
 // rows (phase A), then claims ordinary rows until none are left (phase B).  One
@@ -961,6 +1045,7 @@ __global__ __launch_bounds__(kBlockThreads) void fused_kernel(const Params<IdxT>
    const real_t *tab = stage_table(p.sigmoid_table, lds_tab, (OP >= OP_DOT) && uses_sop && (SOPK >= 0 ? SOPK : p.sop_kind) == SOP_SIGMOID);
    segments_phase<V, L, R, EXACT, OP, SOPK, U, IdxT>(p, tab);
    rows_phase<V, L, R, EXACT, OP, SOPK, U, IdxT>(p, tab);
+   retire_wave<IdxT>(p);
 }
 
 // ---- kernel 3: fold the partials of each heavy row -------------------------------------
@@ -972,8 +1057,7 @@ template <typename IdxT>
 __global__ __launch_bounds__(kBlockThreads) void merge_kernel(const Params<IdxT> p, int generic)
 {
    __shared__ real_t red[kBlockThreads];
-   unsigned int nheavy = p.ctr->n_heavy;
-   if (nheavy > p.cap_heavy) nheavy = p.cap_heavy;
+   const unsigned int nheavy = p.ctr->merge_heavy;   // left by the fused kernel's last workgroup
    const int aop = p.imessage & 0xF0000;
    const int cols = p.k < kBlockThreads ? p.k : kBlockThreads;   // elements handled per pass
    int G = kBlockThreads / cols;                                  // groups (power of two not required)
@@ -1112,26 +1196,41 @@ __global__ __launch_bounds__(kBlockThreads) void zero_rows_kernel(real_t *z, int
       z[(i / k) * ldz + (i % k)] = (real_t)0;
 }
 
-// Clears the queue and claim counters and the queued-row bitmap before each call.
-// A kernel rather than a memset so that callers may capture the stream entry
-// point in a HIP graph.
-__global__ __launch_bounds__(kBlockThreads) void reset_kernel(Counters *c, unsigned int *queued, int64_t words)
-{
-   if (blockIdx.x == 0)
-   {
-      unsigned int *w = reinterpret_cast<unsigned int *>(c);
-      for (unsigned int i = threadIdx.x; i < sizeof(Counters) / sizeof(unsigned int); i += kBlockThreads) w[i] = 0u;
-   }
-   for (int64_t i = (int64_t)blockIdx.x * kBlockThreads + threadIdx.x; i < words; i += (int64_t)gridDim.x * kBlockThreads)
-      queued[i] = 0u;
-}
-
 // Plain 16-byte copy of known size: the yardstick the HBM traffic counters
 // (FETCH_SIZE / WRITE_SIZE) of the kernels above are scaled by.
 __global__ __launch_bounds__(kBlockThreads) void copy_probe_kernel(float4 *dst, const float4 *src, int64_t n16)
 {
    for (int64_t i = (int64_t)blockIdx.x * kBlockThreads + threadIdx.x; i < n16; i += (int64_t)gridDim.x * kBlockThreads)
       dst[i] = src[i];
+}
+
+
+// Read-only stream of known size: every thread keeps U independent 16-byte loads
+// in flight and folds what it read into one word, stored only if it is a value
+// the data never produces, so the loads cannot be dropped and nothing is
+// written.  The yardstick for what this GPU's HBM delivers to reads alone.
+typedef unsigned int probe16_t __attribute__((ext_vector_type(4)));
+template <int U, bool NT>
+__global__ __launch_bounds__(kBlockThreads) void read_probe_kernel(const probe16_t *src, int64_t n16, unsigned int *sink)
+{
+   const int64_t stride = (int64_t)gridDim.x * kBlockThreads;
+   unsigned int acc = 0u;
+   int64_t i = (int64_t)blockIdx.x * kBlockThreads + threadIdx.x;
+   for (; i + (U - 1) * stride < n16; i += U * stride)
+   {
+      probe16_t v[U];
+#pragma unroll
+      for (int u = 0; u < U; u++)
+         v[u] = NT ? __builtin_nontemporal_load(src + i + u * stride) : src[i + u * stride];
+#pragma unroll
+      for (int u = 0; u < U; u++) acc ^= v[u].x ^ v[u].y ^ v[u].z ^ v[u].w;
+   }
+   for (; i < n16; i += stride)
+   {
+      const probe16_t v = src[i];
+      acc ^= v.x ^ v.y ^ v.z ^ v.w;
+   }
+   if (acc == 0x9E3779B9u) *sink = acc;
 }
 
 }  // namespace fmm

@@ -81,8 +81,9 @@ int fusedMM_csr_stream
  * the call allocates and frees nothing.  A call whose queues, sized from m, nnz
  * and k exactly as fusedMM_csr_stream sizes them, do not fit returns
  * FUSEDMM_NOT_ENOUGH_MEM with a message on stderr and touches nothing; so does
- * k > 2048.  (The sigmoid benchmark at K=128 with 2^20 rows and 2^24 edges needs
- * 7.4 MiB.)  Pass the true nnz: it sizes the queues.  The first call on a device
+ * k > 2048 and m > 2^25.  (The first 4 MiB hold the table, the counters and one
+ * bit per row; the sigmoid benchmark at K=128 with 2^20 rows and 2^24 edges needs
+ * 10.9 MiB in all.)  Pass the true nnz: it sizes the queues.  The first call on a device
  * looks up the array's address and copies the 2048-entry table there; do that
  * ahead of time, outside any capture, with fusedMM_amd_init().  All calls on a
  * GPU share the one array: calls enqueued on different streams are ordered one
@@ -138,8 +139,10 @@ int fusedMM_amd_value_bytes(void);
 
 /* 1: pattern-matched tuples use the optimised kernels' write-back rule
  * (default, the reference's ENABLE_OPT_FUSEDMM build, fusedMM.c:512-605);
- * 0: every tuple follows the general pipeline (always accumulates).  Returns
- * the previous setting. */
+ * 0: every tuple follows the general pipeline (always accumulates);
+ * 2: as 1, and a tuple that matches no optimised kernel is refused with
+ * FUSEDMM_NO_OPT_IMPL (the reference built with MUST_OPT_FUSEDMM,
+ * fusedMM.c:599-604).  Returns the previous setting. */
 int fusedMM_amd_set_opt(int enable);
 
 /* 1: before each call, check on the device that every row has pntrb <= pntre
@@ -150,6 +153,24 @@ int fusedMM_amd_set_opt(int enable);
  * previous setting. */
 int fusedMM_amd_set_validate(int enable);
 
+/*
+ * Host-pointer calls (fusedMM_csr with ordinary host arrays) upload every
+ * operand on every call, because the caller may have changed it: the reference
+ * keeps no state either.  fusedMM_amd_set_cache(1) (or FUSEDMM_CACHE=1) keeps a
+ * device mirror of each read-only operand (val, indx, pntrb, pntre, x, y), keyed
+ * by host address and size, and reuses it on later calls; only z then travels.
+ * The caller promises not to change those arrays, or calls
+ * fusedMM_amd_invalidate() after changing them (it drops every mirror; at most
+ * 32 are kept per GPU, the one used longest ago goes first).  Off by default.
+ * Returns the previous setting.
+ */
+int fusedMM_amd_set_cache(int enable);
+void fusedMM_amd_invalidate(void);
+
+/* Upload, kernel and download time in milliseconds of the last fusedMM_csr call
+ * that took host pointers; FUSEDMM_FAIL_RETURN when there was none. */
+int fusedMM_amd_last_host_phases(double *upload_ms, double *kernels_ms, double *download_ms);
+
 /* Tuning knobs of the heavy-row split: rows with more than `heavy_deg` edges
  * are cut into segments of `seg_len` edges (0, 0 restores the K-dependent
  * defaults).  For tests and experiments. */
@@ -157,10 +178,13 @@ void fusedMM_amd_set_split(int64_t heavy_deg, int seg_len);
 
 /*
  * Per-kernel timing with HIP events on the stream the kernels run on.
- * enable != 0 starts a fresh recording (up to 512 calls are kept); the summary
- * waits for the recorded events and returns the number of calls and the summed
- * milliseconds of the three kernels of a call: classify (queues heavy rows),
- * fused (all the gathering and arithmetic), merge (folds split rows).
+ * enable = n > 0 starts a fresh recording of every n-th call (1: every call; up
+ * to 512 calls are kept); 0 stops.  Event records between a call's kernels keep
+ * them from being dispatched back to back (about 20 us per call on an MI355X), so
+ * a caller that also times whole calls samples, e.g. every 4th.  The summary
+ * waits for the recorded events and returns the number of calls recorded and the
+ * summed milliseconds of the three kernels of those calls: classify (queues heavy
+ * rows), fused (all the gathering and arithmetic), merge (folds split rows).
  */
 void fusedMM_amd_timing(int enable);
 int fusedMM_amd_timing_summary(double *classify_ms, double *fused_ms, double *merge_ms);
@@ -176,6 +200,15 @@ int fusedMM_amd_last_split(unsigned int *heavy_rows, unsigned int *segments, uns
  * traffic counters of the kernels are scaled by what they read for this copy
  * of known size. */
 int fusedMM_amd_copy_probe(void *dst, const void *src, int64_t bytes, void *stream);
+
+/* Read `bytes` (a multiple of 16, device memory, 16-byte aligned) with a grid of
+ * blocks_per_cu workgroups per compute unit, each thread keeping `in_flight`
+ * (2, 4, 8 or 16) independent 16-byte loads outstanding, non-temporal or not;
+ * nothing is written (`sink`, 4 bytes of device memory, only keeps the loads
+ * alive).  A measuring aid: what this GPU's HBM delivers to reads alone, next to
+ * which the gather kernels' bandwidth is quoted. */
+int fusedMM_amd_read_probe(const void *src, int64_t bytes, int blocks_per_cu, int in_flight, int nontemporal,
+                           void *sink, void *stream);
 
 /* Release every device buffer the library holds (work queues, staging). */
 void fusedMM_amd_finalize(void);

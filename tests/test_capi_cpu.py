@@ -89,3 +89,46 @@ def test_headers_compile_as_plain_c_and_cpp(tmp_path, compiler, std, idx, val):
                         "-DINDEXTYPE=" + idx, "-DVALUETYPE=" + val, "-I", os.path.join(ROOT, "include"), str(src)],
                        stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
     assert r.returncode == 0, r.stdout
+
+
+def test_must_opt_mode_refuses_unmatched_tuples():
+    """fusedMM_amd_set_opt(2) is the reference built with MUST_OPT_FUSEDMM (fusedMM.c:599-604):
+    a tuple that matches none of the optimised kernels returns FUSEDMM_NO_OPT_IMPL.  Decided
+    from the op tuple alone, before any operand is looked at."""
+    lib = fa.load(32)
+    p = np.zeros(4, np.int32)
+    f = np.zeros(16, np.float32)
+    call = lambda imsg: fa.fusedMM_csr(imsg, 0, 2, 4, 1.0, 0, 2, 2, f, p, p, p, f, 4, f, 4, 0.0, f, 4)
+    prev = lib.fusedMM_amd_set_opt(2)
+    try:
+        assert lib.fusedMM_amd_set_opt(2) == 2
+        for matched in (fa.MSG_GCN, fa.MSG_SPMM, fa.MSG_SIGMOID, fa.MSG_TDIST):
+            assert call(matched) != fa.NO_OPT_IMPL
+        assert call(fa.VOP_ADD | fa.ROP_DOT | fa.SOP_COPY | fa.VSC_MUL | fa.AOP_ADD) == fa.NO_OPT_IMPL
+        assert call(fa.VOP_COPY_RHS | fa.ROP_NOOP | fa.SOP_COPY | fa.VSC_MUL | fa.AOP_MAX) == fa.NO_OPT_IMPL
+        assert call(0x11100) == fa.VOP_FAIL            # a malformed tuple keeps its own code
+        lib.fusedMM_amd_set_opt(1)
+        assert call(fa.VOP_ADD | fa.ROP_DOT | fa.SOP_COPY | fa.VSC_MUL | fa.AOP_ADD) != fa.NO_OPT_IMPL
+    finally:
+        lib.fusedMM_amd_set_opt(prev)
+
+
+def test_cmake_target_of_the_reference_configures(tmp_path):
+    """The consumer project (add_subdirectory + target_link_libraries(... fusedmm), as the
+    reference's CMakeLists.txt:1-14 is used) configures; where the in-tree build exists,
+    its executable really links the library the target names."""
+    import shutil
+    import subprocess
+    if not shutil.which("cmake"):
+        pytest.skip("cmake not installed")
+    src = os.path.join(ROOT, "fusedmm_amd", "consumer")
+    r = subprocess.run(["cmake", "-S", src, "-B", str(tmp_path / "b"), "-DFUSEDMM_INDEX_BITS=32"],
+                       stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True, timeout=120)
+    assert r.returncode == 0, r.stdout
+    r = subprocess.run(["cmake", "--build", str(tmp_path / "b"), "--target", "help"],
+                       stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True, timeout=120)
+    assert "xconsumer" in r.stdout and "fusedmm_build" in r.stdout
+    exe = os.path.join(ROOT, "fusedmm_amd", "cmake_build", "xconsumer")
+    if os.path.exists(exe):
+        r = subprocess.run(["readelf", "-d", exe], stdout=subprocess.PIPE, text=True)
+        assert "libfusedmm.so" in r.stdout

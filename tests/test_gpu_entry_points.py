@@ -250,3 +250,117 @@ def test_nan_dot_product_takes_the_first_table_bin(oracle):
     t0 = oracle.table()[0]
     cols = g["indx"][g["pntrb"][10]:g["pntre"][10]]
     np.testing.assert_allclose(Z[10], ((np.float32(1) - t0) * Y[cols].astype(np.float64)).sum(0), rtol=1e-5, atol=1e-6)
+
+
+def test_cmake_consumer_runs():
+    """The executable the consumer CMake project builds against target `fusedmm`
+    (fusedmm_amd/consumer, built in-tree by __graft_entry__.build()) runs its call on the GPU."""
+    import os
+    import subprocess
+    exe = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), "fusedmm_amd", "cmake_build", "xconsumer")
+    if not os.path.exists(exe):
+        pytest.skip("fusedmm_amd/cmake_build not built")
+    r = subprocess.run([exe], stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True, timeout=120)
+    assert r.returncode == 0 and "PASSED" in r.stdout, r.stdout
+
+
+def test_host_arrays_larger_than_the_pinned_staging_buffers(oracle):
+    """Host-pointer mode moves operands through 16 MiB pinned buffers, a chunk at a
+    time.  Arrays of several chunks and odd sizes arrive and return intact: same bits
+    as the same call on device operands."""
+    n, k = 70001, 132                       # Y and Z: 36.96 MB each, not a multiple of the chunk
+    g = graphs.with_values(graphs.tiny_er(n, 6 * n, 21))
+    X = graphs.features(n, k, 9, -0.5, 0.5, 1)
+    Y = graphs.features(n, k, 9, -0.5, 0.5, 2)
+    Z0 = graphs.features(n, k, 9, -1, 1, 3)
+    gpu_api.set_kind(SOP_NAMES["sigmoid"], 32)
+    for beta in (0.0, 1.0):
+        rc, Zd = gpu_api.run(MSG["s"], g, X, Y, Z0, beta=beta, where="device")
+        assert rc == 0
+        rc, Zh = gpu_api.run(MSG["s"], g, X, Y, Z0, beta=beta, where="host")
+        assert rc == 0
+        np.testing.assert_array_equal(Zh.view(np.uint32), Zd.view(np.uint32))
+    lib = fa.load(32)
+    up, kern, down = C.c_double(), C.c_double(), C.c_double()
+    assert lib.fusedMM_amd_last_host_phases(C.byref(up), C.byref(kern), C.byref(down)) == 0
+    assert up.value > 0 and kern.value > 0 and down.value > 0
+    # X == Y (one buffer): uploaded once, used for both
+    rc, Zd = gpu_api.run(MSG["t"], g, Y, Y, Z0, beta=1.0, where="device")
+    gpu_api.set_kind(SOP_NAMES["tdist"], 32)
+    rc, Zd = gpu_api.run(MSG["t"], g, Y, Y, Z0, beta=1.0, where="device")
+    rc2, Zh = gpu_api.run(MSG["t"], g, Y, Y, Z0, beta=1.0, where="host")
+    assert rc == 0 and rc2 == 0
+    np.testing.assert_array_equal(Zh.view(np.uint32), Zd.view(np.uint32))
+
+
+def test_device_mirrors_of_host_operands_are_opt_in_and_invalidated_on_request():
+    """Default: every host-pointer call re-uploads, so a changed Y is seen.  With
+    fusedMM_amd_set_cache(1) the read-only operands are mirrored on the GPU and a
+    changed Y is NOT seen until fusedMM_amd_invalidate() -- the documented contract."""
+    lib = fa.load(32)
+    g = graphs.with_values(graphs.tiny_er(400, 3000, 8))
+    k = 64
+    Y = graphs.features(400, k, 4, -0.5, 0.5, 2)
+    Z0 = np.zeros((400, k), np.float32)
+    gpu_api.set_kind(0, 32)
+    run = lambda: gpu_api.run(MSG["m"], g, None, Y, Z0, where="host")[1]
+    fresh = lambda: gpu_api.run(MSG["m"], g, None, Y.copy(), Z0, where="device")[1]
+    a = run()
+    Y *= 2.0
+    np.testing.assert_array_equal(run(), fresh())            # default: the change is seen
+    prev = lib.fusedMM_amd_set_cache(1)
+    try:
+        assert prev == 0
+        b = run()                                            # uploads and keeps mirrors
+        np.testing.assert_array_equal(b, fresh())
+        Y *= 0.5                                             # back to the first values, in place
+        np.testing.assert_array_equal(run(), b)              # mirror still holds the doubled Y
+        lib.fusedMM_amd_invalidate()
+        np.testing.assert_array_equal(run(), a)              # re-uploaded
+    finally:
+        lib.fusedMM_amd_set_cache(prev)
+        lib.fusedMM_amd_invalidate()
+
+
+def test_capture_never_reallocates_work_queues(oracle):
+    """Under HIP graph capture fusedMM_csr_stream refuses a call whose work queues
+    would have to grow (replacing them would leave earlier graphs with freed
+    addresses); fusedMM_csr_stream_noalloc takes a size it has never seen, because
+    its queues are the static array.  Replays are checked against eager results,
+    with eager work in between."""
+    import torch
+    lib = fa.load(64)                                         # a library no other test has given big queues
+    assert lib.fusedMM_amd_init() == 0                        # one-time set-up, outside the capture
+    g = graphs.ragged(64, rows=300, cols=4000, hub_deg=9000)
+    k = 256
+    Y = graphs.features(g["cols"], k, 5, -0.5, 0.5, 2)
+    d = dict(val=_dev(g["val"]), indx=_dev(g["indx"]), pb=_dev(g["pntrb"]), pe=_dev(g["pntre"]), Y=_dev(Y))
+    dev = torch.device("cuda:0")
+
+    def enqueue(Z, noalloc, nnz):
+        return fa.fusedMM_csr(fa.MSG_SPMM, g["rows"], g["cols"], k, 1.0, nnz, g["rows"], g["cols"], d["val"], d["indx"],
+                              d["pb"], d["pe"], None, k, d["Y"], k, 0.0, Z, k, index_bits=64,
+                              stream=torch.cuda.current_stream().cuda_stream, noalloc=noalloc)
+
+    Zeager = torch.zeros((g["rows"], k), device=dev)
+    assert enqueue(Zeager, False, g["nnz"]) == 0              # sizes the grown queues for this nnz
+    torch.cuda.synchronize()
+    assert gpu_api.last_split(64)[1] > 0
+    Zg = torch.full((g["rows"], k), 9.0, device=dev)
+    Zn = torch.full((g["rows"], k), 9.0, device=dev)
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        big = enqueue(Zg, False, 50 * g["nnz"])               # would need larger queues: refused, nothing enqueued
+        ok = enqueue(Zg, False, g["nnz"])                     # fits what exists
+        na = enqueue(Zn, True, g["nnz"])                      # static array: nothing to allocate
+    assert big == fa.NOT_ENOUGH_MEM and ok == 0 and na == 0
+    for rep in range(3):
+        Zg.fill_(float(rep))
+        Zn.fill_(float(-rep))
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(Zg, Zeager) and torch.equal(Zn, Zeager), rep
+        Ze2 = torch.zeros_like(Zeager)                        # eager work between replays, both kinds of queues
+        assert enqueue(Ze2, False, g["nnz"]) == 0 and enqueue(Ze2, True, g["nnz"]) == 0
+        torch.cuda.synchronize()
+        assert torch.equal(Ze2, Zeager)
