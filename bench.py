@@ -22,11 +22,24 @@ sys.path.insert(0, ROOT)
 
 PEAK_HBM_GBPS = 8000.0
 
-# HBM bytes per launch of the dominant kernel from rocprofv3 --pmc FETCH_SIZE and
-# WRITE_SIZE, each scaled by the same counter's reading for a plain 1 GiB copy
-# (one summary per workload under profiles/).  Measured, not computed: refreshed
-# whenever the kernel changes.
-MEASURED_TRAFFIC_BYTES = {"c2": 9759204040, "c3": 125575561662, "c4": 129057569729, "c5": 90428018444}
+# HBM bytes per call from rocprofv3 --pmc FETCH_SIZE and WRITE_SIZE, each scaled by
+# the same counter's reading for a plain 1 GiB copy: measured, not computed, and
+# kept in the rocprofv3 summary of each workload under profiles/ (the line
+# "traffic_bytes_per_call: N"), where this reads it.
+PROFILE_OF = {"c2": "fused_kernel_sigmoid_k128_c2.md", "c3": "spmm_k256_c3_rmat22.md",
+              "c3g": "gcn_k256_c3g_rmat22.md", "c4": "tdist_k64_c4_rmat24.md", "c5": "sigmoid_k512_c5_zipf.md"}
+
+
+def measured_traffic_bytes(workload):
+    """(bytes per call, profile file) from the committed rocprofv3 summary, or (None, None)."""
+    name = PROFILE_OF.get(workload)
+    path = os.path.join(ROOT, "profiles", name) if name else None
+    if not path or not os.path.exists(path):
+        return None, None
+    for line in open(path):
+        if line.startswith("traffic_bytes_per_call:"):
+            return int(line.split(":")[1].split()[0]), "profiles/" + name
+    return None, None
 
 WORKLOADS = {
     # name: (description, op letter, K, sop kind)
@@ -69,17 +82,44 @@ def make_workload(name, scale_down=0):
     raise SystemExit("unknown workload %s" % name)
 
 
+def physical_cores():
+    """Physical cores of this host as lscpu counts them (sockets x cores per socket), or None."""
+    import subprocess
+    try:
+        txt = subprocess.run(["lscpu"], stdout=subprocess.PIPE, text=True, timeout=10).stdout
+        f = {}
+        for line in txt.splitlines():
+            if ":" in line:
+                a, b = line.split(":", 1)
+                f[a.strip()] = b.strip()
+        return int(f["Socket(s)"]) * int(f["Core(s) per socket"])
+    except Exception:
+        return None
+
+
+def sample_rows(g, edge_budget):
+    """Leading rows of the graph holding about edge_budget edges (all rows when the graph is smaller)."""
+    rows = g["rows"]
+    if g["nnz"] <= edge_budget:
+        return rows
+    m = int(np.searchsorted(g["pntre"][:rows].astype(np.int64), edge_budget, side="right"))
+    return max(1, min(rows, m))
+
+
 def cpu_baseline(name, g, X, Y, tkern, kind_id, k, budget_s=12.0):
     """The CPU oracle's OpenMP port timed on this host's cores, on a bounded
-    sample of the same workload: the first rows of the graph (m < rows is part
-    of the API).  Checker-side code: used here only to report a baseline."""
+    sample of the same workload: the leading rows of the graph (m < rows is part
+    of the API), all rows when that fits the time budget.  Next to it, on the same
+    sample, the real reference's general fusedMM_csr where oracle/_ref was built.
+    Checker-side code: used here only to report a baseline."""
     sys.path.insert(0, os.path.join(ROOT, "tests"))
-    from oracle_api import Oracle
+    from oracle_api import Oracle, Ref, ref_available
     from fusedmm_amd import synth
     orc = Oracle(fast=True)
     threads = orc.max_threads()
     rows = g["rows"]
-    m = min(rows, 1 << 18)
+    # about 5e7 edges/s on 8 cores at K=128: size the sample for a few calls inside the budget
+    m = sample_rows(g, int(2.5e9 / k))
     nnz_s = int(g["pntre"][m - 1]) - int(g["pntrb"][0])
     Z = np.zeros((m, k), np.float32)
     ot = "t" if tkern == "f" else tkern
@@ -92,11 +132,37 @@ def cpu_baseline(name, g, X, Y, tkern, kind_id, k, budget_s=12.0):
         t_all.append(time.time() - t1)
     t = float(np.mean(t_all))
     flops = synth.algorithmic_flops(tkern, k, nnz_s)
-    return {"value": flops / t / 1e9, "unit": "GFLOP/s", "cores": threads, "kind": "port",
-            "sample": "first %d of %d rows of the same workload (%d edges), %d calls, mean %.4f s/call"
-                      % (m, rows, nnz_s, len(t_all), t),
-            "edges_per_s": nnz_s / t,
-            "alg_GBps": synth.algorithmic_bytes(tkern, m, k, nnz_s) / t / 1e9}
+    out = {"value": flops / t / 1e9, "unit": "GFLOP/s", "cores": threads, "kind": "port",
+           "sample": "first %d of %d rows of the same workload (%d of %d edges), %d calls, mean %.4f s/call; "
+                     "OpenMP restatement built -O3 -march=x86-64-v3 (AVX2+FMA, not the host's widest ISA)"
+                     % (m, rows, nnz_s, g["nnz"], len(t_all), t),
+           "omp_max_threads": threads, "lscpu_physical_cores": physical_cores(),
+           "edges_per_s": nnz_s / t,
+           "alg_GBps": synth.algorithmic_bytes(tkern, m, k, nnz_s) / t / 1e9}
+    # the real reference's general pipeline (fusedMM.c compiled where it lies, 8 OpenMP threads as its
+    # build fixes them) on the same rows: lets a reader relate the port to the reference on this host
+    ref_kind = {"s": "sigmoid", "t": "tdist", "f": "fr", "m": "spmm", "g": "gcn"}[tkern]
+    if ref_available(ref_kind, 32, 32):
+        from oracle_api import MSG
+        ref = Ref(ref_kind, 32, 32)
+        Zr = np.zeros((m, k), np.float32)
+        Xr = X if X is not None else Y
+        ref.fusedMM_csr(MSG[tkern], g, Xr, Y, Zr, 0.0, m=m)       # warm-up
+        tr = []
+        t0 = time.time()
+        while (len(tr) < 2 or time.time() - t0 < 0.6 * budget_s) and len(tr) < 50:
+            Zr[:] = 0
+            t1 = time.time()
+            ref.fusedMM_csr(MSG[tkern], g, Xr, Y, Zr, 0.0, m=m)
+            tr.append(time.time() - t1)
+        tm = float(np.mean(tr))
+        out["reference_general"] = {"kind": "reference-general", "value": flops / tm / 1e9, "unit": "GFLOP/s",
+                                    "cores": 8, "edges_per_s": nnz_s / tm,
+                                    "sample": "same rows; the reference's general fusedMM_csr (five indirect stage calls "
+                                              "per edge, NTHREADS=8 fixed at build time), %d calls, mean %.4f s/call; "
+                                              "its optimised kernels need its code generator and are not built here"
+                                              % (len(tr), tm)}
+    return out
 
 
 def main():
@@ -111,6 +177,12 @@ def main():
     ap.add_argument("--no-check", action="store_true", help="skip the spot check against the oracle")
     ap.add_argument("--copy-probe", action="store_true",
                     help="also launch a plain 1 GiB copy kernel (yardstick for rocprofv3 --pmc FETCH_SIZE/WRITE_SIZE)")
+    ap.add_argument("--kernel-events-every", type=int, default=4,
+                    help="record per-kernel HIP events on every n-th timed step (0: none).  An event record between "
+                         "two kernels keeps them from being dispatched back to back, about 20 us per step, so the "
+                         "timed region samples rather than instruments every step")
+    ap.add_argument("--read-probe", action="store_true",
+                    help="also time a read-only stream over 4 GiB (what HBM delivers to reads alone) and report it")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py: this path is built and measured on ONE GPU; --gpus %d is not supported "
@@ -162,10 +234,29 @@ def main():
         torch.cuda.synchronize()
         del src, dst
 
+    read_probe = None
+    if args.read_probe:
+        nbytes = 4 << 30
+        src = torch.empty(nbytes // 4, dtype=torch.float32, device=dev).uniform_(-1, 1)
+        sink = torch.zeros(4, dtype=torch.int32, device=dev)
+        read_probe = {"bytes": nbytes}
+        for label, nt in (("plain_loads", 0), ("nontemporal_loads", 1)):
+            for _ in range(2):
+                assert lib.fusedMM_amd_read_probe(src.data_ptr(), nbytes, 16, 8, nt, sink.data_ptr(), stream) == 0
+            torch.cuda.synchronize()
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record()
+            for _ in range(10):
+                lib.fusedMM_amd_read_probe(src.data_ptr(), nbytes, 16, 8, nt, sink.data_ptr(), stream)
+            e1.record()
+            torch.cuda.synchronize()
+            read_probe[label + "_GBps"] = nbytes / (e0.elapsed_time(e1) / 10 * 1e-3) / 1e9
+        del src, sink
+
     for _ in range(args.warmup):
         step()
     torch.cuda.synchronize()
-    lib.fusedMM_amd_timing(1)
+    lib.fusedMM_amd_timing(max(0, args.kernel_events_every))
     t0 = time.perf_counter()
     for _ in range(args.steps):
         step()
@@ -189,16 +280,22 @@ def main():
                "merge_kernel": g_ms.value / max(1, ncalls)}
     # dominant kernel: fused_kernel does all the gathering.  When rows were split, the
     # partial results it writes are folded by merge_kernel, so the call's algorithmic
-    # bytes are quoted on the two together (classify_kernel only reads row pointers).
+    # bytes are quoted on the three together (classify_kernel only reads row pointers).
     hs = (C.c_uint(), C.c_uint(), C.c_uint())
     lib.fusedMM_amd_last_split(C.byref(hs[0]), C.byref(hs[1]), C.byref(hs[2]))
     split = hs[1].value > 0
     dom_ms = kern_ms["fused_kernel"] + (kern_ms["merge_kernel"] + kern_ms["classify_kernel"] if split else 0.0)
+    if ncalls <= 0:
+        dom_ms = ms_per_step      # no step carried events: whole-step wall time stands in (an upper bound)
     achieved = b_alg / (dom_ms * 1e-3) / 1e9 if dom_ms > 0 else 0.0
+    traffic, traffic_from = measured_traffic_bytes(args.workload) if vbits == 32 else (None, None)
     roofline = {"bound": "hbm", "achieved": achieved, "peak": PEAK_HBM_GBPS, "unit": "GB/s",
-                "frac": achieved / PEAK_HBM_GBPS, "traffic": MEASURED_TRAFFIC_BYTES.get(args.workload) if vbits == 32 else None,
+                "frac": achieved / PEAK_HBM_GBPS, "traffic": traffic, "traffic_from": traffic_from,
                 "kernel": "classify_kernel+fused_kernel+merge_kernel" if split else "fused_kernel",
                 "kernel_ms": dom_ms, "algorithmic_bytes": b_alg}
+    if read_probe:
+        roofline["read_stream_probe"] = read_probe
+        roofline["frac_of_read_stream"] = achieved / read_probe["plain_loads_GBps"]
 
     checked = None
     if not args.no_check:
@@ -237,6 +334,7 @@ def main():
         "hbm_GBps_algorithmic": b_alg / (ms_per_step * 1e-3) / 1e9,
         "pct_peak_hbm": 100.0 * b_alg / (ms_per_step * 1e-3) / 1e9 / PEAK_HBM_GBPS,
         "kernel_ms": kern_ms,
+        "kernel_events": {"every_nth_step": args.kernel_events_every, "steps_recorded": max(0, ncalls)},
         "kernels_ms_per_call": {"min": float(np.min(per_call)), "median": float(np.median(per_call)),
                                 "max": float(np.max(per_call))} if per_call else None,
         "split": {"heavy_rows": hs[0].value, "segments": hs[1].value, "overflow": hs[2].value},
@@ -245,6 +343,12 @@ def main():
     }
     if not args.no_cpu and vbits == 32:
         out["cpu_baseline"] = cpu_baseline(args.workload, g, X, Y, tkern, kind_id, k)
+    if checked is False:
+        # a run whose output differs from the oracle's is not a measurement
+        out["value"] = None
+        out["error"] = "spot check against the oracle failed: results differ"
+        print(json.dumps(out))
+        sys.exit(3)
     print(json.dumps(out))
 
 
