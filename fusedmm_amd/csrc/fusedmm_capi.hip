@@ -356,7 +356,10 @@ int launch_instance(const Params<idx_t> &p, const Launch &l)
    if (l.ev) FMM_HIP(hipEventRecord(l.ev[1], l.stream));
    hipLaunchKernelGGL((fused_kernel<V, L, R, EXACT, OP, SOPK, U, idx_t>), dim3((unsigned int)gr), dim3(kBlockThreads), 0, l.stream, pr);
    if (l.ev) FMM_HIP(hipEventRecord(l.ev[2], l.stream));
-   hipLaunchKernelGGL((merge_kernel<idx_t>), dim3((unsigned int)(l.num_cu * 2)), dim3(kBlockThreads), 0, l.stream, p, (int)(OP == OP_GENERIC));
+   // one workgroup per heavy row and pass of 256 columns
+   const unsigned int col_passes = (unsigned int)((p.k + kBlockThreads - 1) / kBlockThreads);
+   hipLaunchKernelGGL((merge_kernel<idx_t>), dim3((unsigned int)(l.num_cu * 2), col_passes), dim3(kBlockThreads), 0, l.stream,
+                      p, (int)(OP == OP_GENERIC));
    if (l.ev) FMM_HIP(hipEventRecord(l.ev[3], l.stream));
    return hip_status(hipGetLastError(), "kernel launch");
 }

@@ -56,8 +56,8 @@ constexpr int kWavesPerBlock = kBlockThreads / 64;
 // finish puts them back (and clears the queued-row bits), so a call needs no
 // reset pass of its own.
 struct Counters {
-   unsigned int n_heavy;    // heavy rows queued by the classify kernel
-   unsigned int n_seg;      // edge segments queued
+   unsigned int n_heavy;    // heavy rows queued by the classify kernel   } advanced together, as one
+   unsigned int n_seg;      // edge segments queued                       } 64-bit word (n_heavy low)
    unsigned int overflow;   // heavy rows that did not fit the queue (processed whole in phase B)
    unsigned int done_groups; // groups of workgroups of the fused kernel that have finished (see retire[])
    unsigned int invalid;    // set by the optional operand check
@@ -741,17 +741,38 @@ __device__ __forceinline__ int64_t resolve_claim(const Params<IdxT> &p, unsigned
 template <typename IdxT>
 __global__ __launch_bounds__(kBlockThreads) void classify_kernel(const Params<IdxT> p)
 {
+   const int lane = threadIdx.x & 63;
    const int64_t stride = (int64_t)gridDim.x * kBlockThreads;
-   for (int64_t row = (int64_t)blockIdx.x * kBlockThreads + threadIdx.x; row < p.m; row += stride)
-   {
-      const IdxT jb = p.pntrb[row];
-      const int64_t deg = (int64_t)p.pntre[row] - (int64_t)jb;
-      if (deg <= p.heavy_deg) continue;
+   // Queue entries are handed out by ONE 64-bit read-modify-write per wavefront and
+   // turn: n_heavy (low word) and n_seg (high word) advance together, by the number of
+   // heavy rows among the wave's 64 rows and by the sum of their segment counts.  Every
+   // heavy row taking the two counters by itself made this pass wait ~12 ns per
+   // read-modify-write on the one cache line (13 000 heavy rows of an R-MAT graph: 0.2 ms).
+   unsigned long long *both = reinterpret_cast<unsigned long long *>(&p.ctr->n_heavy);
+   auto queue_rows = [&](int64_t row, IdxT jb, IdxT je) {
+      const int64_t deg = (int64_t)je - (int64_t)jb;
+      const bool heavy = deg > p.heavy_deg;
+      const unsigned long long mask = __ballot(heavy);
+      if (mask == 0ull) return;                                    // wave-uniform
       int64_t seg_len = p.seg_len;
       if (deg > seg_len * (int64_t)kMaxSegsPerRow) seg_len = (deg + kMaxSegsPerRow - 1) / kMaxSegsPerRow;
-      const unsigned int nseg = (unsigned int)((deg + seg_len - 1) / seg_len);
-      const unsigned int slot = atomicAdd(&p.ctr->n_heavy, 1u);
-      const unsigned int base = atomicAdd(&p.ctr->n_seg, nseg);
+      const unsigned int nseg = heavy ? (unsigned int)((deg + seg_len - 1) / seg_len) : 0u;
+      unsigned int incl = nseg;                                    // inclusive prefix sum of nseg over the lanes
+#pragma unroll
+      for (int d = 1; d < 64; d <<= 1)
+      {
+         const unsigned int up = __shfl_up(incl, d, 64);
+         if (lane >= d) incl += up;
+      }
+      const unsigned int total = __shfl(incl, 63, 64);
+      const int leader = __builtin_ctzll(mask);
+      unsigned long long before = 0ull;
+      if (lane == leader)
+         before = atomicAdd(both, (unsigned long long)__builtin_popcountll(mask) | ((unsigned long long)total << 32));
+      before = __shfl(before, leader, 64);
+      if (!heavy) return;
+      const unsigned int slot = (unsigned int)(before & 0xFFFFFFFFull) + (unsigned int)__builtin_popcountll(mask & ((1ull << lane) - 1ull));
+      const unsigned int base = (unsigned int)(before >> 32) + (incl - nseg);
       if (slot < p.cap_heavy && (uint64_t)base + nseg <= (uint64_t)p.cap_seg)
       {
          p.heavy[slot] = HeavyRow{row, base, nseg};
@@ -772,6 +793,23 @@ __global__ __launch_bounds__(kBlockThreads) void classify_kernel(const Params<Id
          for (uint64_t s = base; s < (uint64_t)base + nseg && s < (uint64_t)p.cap_seg; s++)
             p.segs[s] = SegDesc{-1, 0, 0u, 0u};
       }
+   };
+   // four rows per thread and turn, their pointers requested together; the turn's
+   // bounds are the wave's (its first lane's row), so that every lane takes part in
+   // the wave-wide steps above
+   constexpr int kRowsPerTurn = 4;
+   for (int64_t row0 = (int64_t)blockIdx.x * kBlockThreads + threadIdx.x; row0 - lane < p.m; row0 += kRowsPerTurn * stride)
+   {
+      IdxT jb[kRowsPerTurn], je[kRowsPerTurn];
+#pragma unroll
+      for (int i = 0; i < kRowsPerTurn; i++)
+      {
+         const int64_t row = row0 + i * stride;
+         jb[i] = row < p.m ? p.pntrb[row] : (IdxT)0;
+         je[i] = row < p.m ? p.pntre[row] : (IdxT)0;
+      }
+#pragma unroll
+      for (int i = 0; i < kRowsPerTurn; i++) queue_rows(row0 + i * stride, jb[i], je[i]);
    }
 }
 
@@ -1069,7 +1107,8 @@ __global__ __launch_bounds__(kBlockThreads) void merge_kernel(const Params<IdxT>
       const HeavyRow hr = p.heavy[h];
       if (hr.n_seg == 0) continue;
       real_t *zrow = p.z + hr.row * p.ldz;
-      for (int e0 = 0; e0 < p.k; e0 += cols)
+      // columns in passes of `cols`, the passes dealt to the grid's second dimension
+      for (int e0 = (int)blockIdx.y * cols; e0 < p.k; e0 += (int)gridDim.y * cols)
       {
          const int e = e0 + col;
          const bool live = active && e < p.k;
@@ -1081,6 +1120,15 @@ __global__ __launch_bounds__(kBlockThreads) void merge_kernel(const Params<IdxT>
             unsigned int s = grp;
             if (!is_max && !is_min)
             {
+               // 16 partials requested at a time, added in ascending order as before
+               for (; s + 15u * G < hr.n_seg; s += 16u * G)
+               {
+                  real_t v[16];
+#pragma unroll
+                  for (unsigned int i = 0; i < 16u; i++) v[i] = pp[(int64_t)(s + i * G) * p.kpad];
+#pragma unroll
+                  for (unsigned int i = 0; i < 16u; i++) a += v[i];
+               }
                for (; s + 3u * G < hr.n_seg; s += 4u * G)
                {
                   const real_t v0 = pp[(int64_t)s * p.kpad], v1 = pp[(int64_t)(s + G) * p.kpad],

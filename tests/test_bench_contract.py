@@ -36,3 +36,24 @@ def test_scaled_workloads_have_the_advertised_shape():
     assert X is Y and np.abs(X).max() <= 1.0                          # A = B, U[-1, 1]
     g, _, _ = bench.make_workload("c5", 6)
     assert np.diff(g["rowptr"]).max() == min(1000000, (1 << 15) // 2)  # hubs at the cap
+
+
+def test_traffic_figures_come_from_the_committed_profiles():
+    """roofline.traffic is read from the rocprofv3 summary of the workload (no table
+    in bench.py to go stale): every profiled workload has a parsable figure that sits
+    next to the algorithmic bytes the same file states."""
+    import re
+    sys.path.insert(0, ROOT)
+    import bench
+    for w, fname in bench.PROFILE_OF.items():
+        path = os.path.join(ROOT, "profiles", fname)
+        assert os.path.exists(path), fname
+        got, src = bench.measured_traffic_bytes(w)
+        assert src == "profiles/" + fname and got and got > 0
+        text = open(path).read()
+        m = re.search(r"traffic per call: ([0-9.]+) GB against ([0-9.]+) GB algorithmic", text)
+        assert m, fname
+        assert abs(got / 1e9 - float(m.group(1))) < 1e-3
+        assert 0.8 < got / 1e9 / float(m.group(2)) < 1.1, (w, got)
+        assert "rocprofv3 --kernel-trace --stats" in text and "python3 bench.py --workload " + w in text
+    assert bench.measured_traffic_bytes("c1") == (None, None)      # cache-resident case: no roofline claim
