@@ -102,6 +102,9 @@ struct DeviceState {
    hipEvent_t order_ev[2];
    hipStream_t last_stream[2] = {nullptr, nullptr};
    bool pending[2] = {false, false};
+   // A call whose kernels could not all be launched may leave counters or queued-row
+   // bits set; the next call on these queues then clears them before it starts.
+   bool dirty[2] = {false, false};
    Counters *last_ctr = nullptr;   // counters of the most recent call (fusedMM_amd_last_split)
    // timing
    hipEvent_t ev[kTimingSlots][4];   // around the three kernels of a call
@@ -594,6 +597,18 @@ int run_slab(const Args &a, const Plan &pl, int sop_kind, hipStream_t stream, in
    p.cap_heavy = (unsigned int)cap_heavy;
    p.cap_seg = (unsigned int)cap_seg;
    d->last_ctr = p.ctr;
+   if (d->dirty[queues])
+   {
+      if (capturing)
+      {
+         FMM_LOG("an earlier call failed part-way; call once outside the capture (or fusedMM_amd_finalize()) first");
+         return FUSEDMM_FAIL_RETURN;
+      }
+      FMM_HIP(hipDeviceSynchronize());
+      FMM_HIP(hipMemset(p.ctr, 0, sizeof(Counters)));
+      FMM_HIP(hipMemset(p.queued, 0, queues == kQueuesStatic ? (size_t)(kScratchMaxRows / 8) : d->queued.bytes));
+      d->dirty[queues] = false;
+   }
 
    // Calls that share these queues must run one after the other.  On one stream
    // they do; a call on another stream first waits for what the previous call's
@@ -639,7 +654,11 @@ int run_slab(const Args &a, const Plan &pl, int sop_kind, hipStream_t stream, in
          break;
       default: st = launch_op<OP_GENERIC, -1>(p, sh, l); break;
    }
-   if (st) return st;
+   if (st)
+   {
+      d->dirty[queues] = true;
+      return st;
+   }
    if (!capturing)
    {
       d->pending[queues] = true;
