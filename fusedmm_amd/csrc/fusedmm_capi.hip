@@ -1488,6 +1488,18 @@ void fusedMM_amd_timing(int enable)
    g.timing = enable > 0 ? enable : 0;
    g.timing_seen = 0;
    g.timing_calls = 0;
+   if (g.timing > 0)
+   {
+      // the events are made here, on the current device, not inside the first timed call
+      DeviceState *d = nullptr;
+      if (device_basics(&d) == FUSEDMM_SUCCESS_RETURN && !d->ev_made)
+      {
+         bool ok = true;
+         for (int i = 0; i < kTimingSlots && ok; i++)
+            for (int e = 0; e < 4 && ok; e++) ok = (hipEventCreate(&d->ev[i][e]) == hipSuccess);
+         d->ev_made = ok;
+      }
+   }
 }
 
 int fusedMM_amd_timing_summary(double *classify_ms, double *fused_ms, double *merge_ms)

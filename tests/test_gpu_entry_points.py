@@ -364,3 +364,51 @@ def test_capture_never_reallocates_work_queues(oracle):
         assert enqueue(Ze2, False, g["nnz"]) == 0 and enqueue(Ze2, True, g["nnz"]) == 0
         torch.cuda.synchronize()
         assert torch.equal(Ze2, Zeager)
+
+
+def test_two_host_threads_calling_at_once(oracle):
+    """The entry points may be called from several host threads (the reference is
+    re-entrant); the library serialises the enqueueing and orders the calls on the
+    GPU.  Each thread uses its own stream, operands and output; every result must
+    equal the single-threaded one."""
+    import threading
+    import torch
+    g = graphs.ragged(32, rows=400, cols=6000, hub_deg=20000)
+    k = 64
+    X = graphs.features(g["rows"], k, 3, -0.5, 0.5, 1)
+    Ys = [graphs.features(g["cols"], k, 30 + i, -0.5, 0.5, 2) for i in range(3)]
+    d = dict(val=_dev(g["val"]), indx=_dev(g["indx"]), pb=_dev(g["pntrb"]), pe=_dev(g["pntre"]), X=_dev(X))
+    dY = [_dev(y) for y in Ys]
+    gpu_api.set_kind(SOP_NAMES["sigmoid"], 32)
+
+    def enqueue(Y, Z, stream):
+        return fa.fusedMM_csr(fa.MSG_SIGMOID, g["rows"], g["cols"], k, 1.0, g["nnz"], g["rows"], g["cols"], d["val"],
+                              d["indx"], d["pb"], d["pe"], d["X"], k, Y, k, 0.0, Z, k, stream=stream)
+
+    want = []
+    for y in dY:
+        Z = torch.zeros((g["rows"], k), device="cuda:0")
+        assert enqueue(y, Z, torch.cuda.current_stream().cuda_stream) == 0
+        torch.cuda.synchronize()
+        want.append(Z)
+    streams = [torch.cuda.Stream() for _ in dY]
+    got = [[torch.full((g["rows"], k), 3.0, device="cuda:0") for _ in range(20)] for _ in dY]
+    errors = []
+
+    def worker(i):
+        for rep in range(20):
+            rc = enqueue(dY[i], got[i][rep], streams[i].cuda_stream)
+            if rc != 0:
+                errors.append((i, rep, rc))
+
+    torch.cuda.synchronize()
+    threads = [threading.Thread(target=worker, args=(i,)) for i in range(len(dY))]
+    for t in threads:
+        t.start()
+    for t in threads:
+        t.join()
+    torch.cuda.synchronize()
+    assert not errors, errors
+    for i in range(len(dY)):
+        for rep in range(20):
+            assert torch.equal(got[i][rep], want[i]), (i, rep)
