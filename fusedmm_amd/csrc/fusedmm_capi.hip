@@ -501,11 +501,20 @@ int run_slab(const Args &a, const Plan &pl, int sop_kind, hipStream_t stream, in
       return FUSEDMM_FAIL_RETURN;
    }
    DeviceState *d = nullptr;
-   int st = (queues == kQueuesStatic) ? device_basics(&d) : device_state(&d);
+   int st = device_basics(&d);
    if (st) return st;
-   if (queues == kQueuesStatic) { st = scratch_setup(*d); if (st) return st; }
    bool capturing = false;
    st = stream_capturing(stream, &capturing);
+   if (st) return st;
+   // First use on a device copies the sigmoid table and clears the counters with
+   // blocking calls (and, for the grown queues, allocates): not while a capture is open.
+   if (capturing && (queues == kQueuesStatic ? d->scratch == nullptr : !d->ready))
+   {
+      FMM_LOG("first use on this device while the stream is being captured; call fusedMM_amd_init() before the capture");
+      return FUSEDMM_FAIL_RETURN;
+   }
+   if (queues == kQueuesStatic) st = scratch_setup(*d);
+   else st = device_state(&d);
    if (st) return st;
 
    // 16-byte accesses need 16-byte aligned rows: leading dimensions a multiple of 4 floats / 2 doubles
@@ -1295,6 +1304,16 @@ int entry(const Args &a, bool async, hipStream_t stream, int queues = kQueuesGro
       if (a.m <= 0 || a.k < 1) return FUSEDMM_SUCCESS_RETURN;
       if (g.validate)
       {
+         // the check reads a flag back and waits for it: impossible inside a capture
+         bool capturing = false;
+         st = stream_capturing(stream, &capturing);
+         if (st) return st;
+         if (capturing)
+         {
+            FMM_LOG("operand validation is switched on and the stream is being captured; "
+                    "validate once outside the capture, then switch it off (fusedMM_amd_set_validate(0))");
+            return FUSEDMM_FAIL_RETURN;
+         }
          st = validate_operands(a, stream, queues);
          if (st) return st;
       }

@@ -102,8 +102,12 @@ int64_t fusedMM_amd_noalloc_capacity(void);
 
 /* Set up the current device ahead of the first call: small fixed allocations of
  * the ordinary entry points (sigmoid table, counters) and the static array of
- * fusedMM_csr_stream_noalloc.  Optional; every entry point does its part of this
- * on first use.  Returns a fusedMM status code. */
+ * fusedMM_csr_stream_noalloc.  Optional outside HIP graph capture, where every
+ * entry point does its part of this on first use; required before a device's
+ * first call is captured (that call returns FUSEDMM_FAIL_RETURN otherwise, as the
+ * set-up copies and clears with blocking calls).  Operand validation
+ * (fusedMM_amd_set_validate) waits for the GPU too: a captured call is refused
+ * while it is switched on.  Returns a fusedMM status code. */
 int fusedMM_amd_init(void);
 
 /*

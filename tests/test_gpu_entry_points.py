@@ -322,6 +322,56 @@ def test_device_mirrors_of_host_operands_are_opt_in_and_invalidated_on_request()
         lib.fusedMM_amd_invalidate()
 
 
+def test_capture_refuses_what_would_block(oracle):
+    """A device's first call (blocking set-up copies, allocations) and a call with operand
+    validation switched on (reads a flag back) cannot be recorded into a HIP graph: both
+    are refused with FUSEDMM_FAIL_RETURN before anything is enqueued, and the same calls
+    succeed once the set-up has been done outside the capture and validation is off."""
+    import torch
+    lib = fa.load(64)
+    g = graphs.with_values(graphs.tiny_er(300, 2000, 21, bits=64))
+    k = 32
+    Y = graphs.features(300, k, 6, -0.5, 0.5, 2)
+    d = dict(val=_dev(g["val"]), indx=_dev(g["indx"]), pb=_dev(g["pntrb"]), pe=_dev(g["pntre"]), Y=_dev(Y))
+    dev = torch.device("cuda:0")
+
+    def enqueue(Z, noalloc):
+        return fa.fusedMM_csr(fa.MSG_SPMM, g["rows"], g["cols"], k, 1.0, g["nnz"], g["rows"], g["cols"], d["val"], d["indx"],
+                              d["pb"], d["pe"], None, k, d["Y"], k, 0.0, Z, k, index_bits=64,
+                              stream=torch.cuda.current_stream().cuda_stream, noalloc=noalloc)
+
+    torch.cuda.synchronize()
+    lib.fusedMM_amd_finalize()                                # this library now knows nothing of the device
+    Z1 = torch.full((g["rows"], k), 7.0, device=dev)
+    Z2 = torch.full((g["rows"], k), 7.0, device=dev)
+    Zwarm = torch.zeros((g["rows"], k), device=dev)
+    first = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(first):
+        rc_grown = enqueue(Z1, False)
+        rc_static = enqueue(Z2, True)
+        Zwarm.add_(1.0)                                       # something to record, so the graph is not empty
+    assert rc_grown == fa.FAIL and rc_static == fa.FAIL
+    assert lib.fusedMM_amd_init() == 0
+    Zeager = torch.zeros((g["rows"], k), device=dev)
+    assert enqueue(Zeager, False) == 0                        # sizes the grown queues
+    torch.cuda.synchronize()
+    second = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(second):
+        prev = lib.fusedMM_amd_set_validate(1)
+        rc_val = enqueue(Z1, False)
+        rc_val_static = enqueue(Z2, True)
+        lib.fusedMM_amd_set_validate(prev)
+        rc_ok = enqueue(Z1, False)
+        rc_ok_static = enqueue(Z2, True)
+    assert rc_val == fa.FAIL and rc_val_static == fa.FAIL and rc_ok == 0 and rc_ok_static == 0
+    for rep in range(2):
+        Z1.fill_(float(rep) + 2.0)
+        Z2.fill_(float(rep) + 3.0)
+        second.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(Z1, Zeager) and torch.equal(Z2, Zeager), rep
+
+
 def test_capture_never_reallocates_work_queues(oracle):
     """Under HIP graph capture fusedMM_csr_stream refuses a call whose work queues
     would have to grow (replacing them would leave earlier graphs with freed
