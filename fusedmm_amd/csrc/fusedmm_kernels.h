@@ -492,12 +492,14 @@ __device__ __forceinline__ real_t vop_rop(Slice<R> &t, const Slice<R> &xs, const
    return scal;
 }
 
-// The per-edge pipeline: T = VOP(x, y); s = ROP(x, T); d = SOP(s); T = MOP(d, T);
-// acc = AOP(acc, T).  `xs` is the X[i] slice, `ys` the gathered Y[c] slice.
+// One edge of the four optimised tuples: T = VOP(x, y); s = ROP(x, T); d = SOP(s);
+// acc += d * T, fused.  `xs` is the X[i] slice, `ys` the gathered Y[c] slice.  (The
+// general pipeline is general_steps below.)
 template <int L, int R, int OP>
 __device__ __forceinline__ void edge_step(Slice<R> &acc, const Slice<R> &xs, const Slice<R> &ys,
-                                          real_t edge_val, int sop_kind, int imsg, const real_t *tab)
+                                          real_t edge_val, int sop_kind, const real_t *tab)
 {
+   static_assert(OP != OP_GENERIC, "the general pipeline goes through general_steps");
    if (OP == OP_GCN)
    {
 #pragma unroll
@@ -527,35 +529,172 @@ __device__ __forceinline__ void edge_step(Slice<R> &acc, const Slice<R> &xs, con
       const real_t d = sop_eval(sop_kind, s, tab);
       axpy_slice<R>(acc, d, t);
    }
-   else
+}
+
+// The general pipeline over the U edges a sub-wave has in flight, stage by stage:
+// each stage's switch on the op tuple is taken once for the batch, and inside a case
+// the U edges are straight-line code (their reductions and table look-ups overlap).
+// Arithmetic and order of accumulation are those of edge_step, edge 0 first; edges
+// with ok[u] false change nothing.  ys[u] is overwritten with T.
+template <int L, int R, int U>
+__device__ __forceinline__ void general_steps(Slice<R> &acc, const Slice<R> &xs, Slice<R> *ys, const real_t *ev,
+                                              const bool *ok, int sop_kind, int imsg, const real_t *tab)
+{
+   const int vop = imsg & 0xF, rop = imsg & 0xF0, sop = imsg & 0xF00, vsc = imsg & 0xF000, aop = imsg & 0xF0000;
+#define FMM_EACH_EDGE for (int u = 0; u < U; u++)
+   switch (vop)
    {
-      const int vop = imsg & 0xF, rop = imsg & 0xF0, sop = imsg & 0xF00, vsc = imsg & 0xF000,
-                aop = imsg & 0xF0000;
-      Slice<R> t;
-      const real_t scal = vop_rop<L, R>(t, xs, ys, edge_val, vop, rop);
-      const real_t d = (sop == kSopUdef) ? sop_eval(sop_kind, scal, tab) : scal;
-      if (vsc == kVscMul)
-      {
+      case kVopCopyLhs:
 #pragma unroll
-         for (int r = 0; r < R; r++)
-         {
-            t.v[r].x = d * t.v[r].x; t.v[r].y = d * t.v[r].y;
-            t.v[r].z = d * t.v[r].z; t.v[r].w = d * t.v[r].w;
-         }
-      }
-      else if (vsc == kVscAdd)
-      {
+         FMM_EACH_EDGE ys[u] = xs;
+         break;
+      case kVopCopyRhs: break;
+      case kVopAdd:
 #pragma unroll
-         for (int r = 0; r < R; r++)
-         {
-            t.v[r].x = d + t.v[r].x; t.v[r].y = d + t.v[r].y;
-            t.v[r].z = d + t.v[r].z; t.v[r].w = d + t.v[r].w;
-         }
-      }
-      if (aop == kAopAdd) map2(acc, acc, t, [](real_t a, real_t b) { return a + b; });
-      else if (aop == kAopMax) map2(acc, acc, t, [](real_t a, real_t b) { return a > b ? a : b; });
-      else if (aop == kAopMin) map2(acc, acc, t, [](real_t a, real_t b) { return a < b ? a : b; });
+         FMM_EACH_EDGE map2(ys[u], xs, ys[u], [](real_t a, real_t b) { return a + b; });
+         break;
+      case kVopSubl:
+#pragma unroll
+         FMM_EACH_EDGE map2(ys[u], xs, ys[u], [](real_t a, real_t b) { return -a + b; });
+         break;
+      case kVopSubr:
+#pragma unroll
+         FMM_EACH_EDGE map2(ys[u], xs, ys[u], [](real_t a, real_t b) { return a - b; });
+         break;
+      case kVopMax:
+#pragma unroll
+         FMM_EACH_EDGE map2(ys[u], xs, ys[u], [](real_t a, real_t b) { return a > b ? a : b; });
+         break;
+      default:
+#pragma unroll
+         FMM_EACH_EDGE map2(ys[u], xs, ys[u], [](real_t a, real_t b) { return a < b ? a : b; });
+         break;
    }
+   real_t d[U];
+#pragma unroll
+   FMM_EACH_EDGE d[u] = ev[u];
+   switch (rop)
+   {
+      case kRopDot:
+#pragma unroll
+         FMM_EACH_EDGE d[u] = dot_slices<L, R>(xs, ys[u]);
+         break;
+      case kRopAddLhs:
+      {
+         const real_t sx = sum_slice<L, R>(xs);
+#pragma unroll
+         FMM_EACH_EDGE d[u] = sx;
+         break;
+      }
+      case kRopAddRhs:
+#pragma unroll
+         FMM_EACH_EDGE d[u] = sum_slice<L, R>(ys[u]);
+         break;
+      case kRopNormL:
+      {
+         const real_t nx = dot_slices<L, R>(xs, xs);
+#pragma unroll
+         FMM_EACH_EDGE d[u] = nx;
+         break;
+      }
+      case kRopNormR:
+#pragma unroll
+         FMM_EACH_EDGE d[u] = dot_slices<L, R>(ys[u], ys[u]);
+         break;
+      default: break;
+   }
+   if (sop == kSopUdef)
+   {
+      switch (sop_kind)
+      {
+#define FMM_SOP_CASE(K_)                                 \
+   case K_:                                              \
+      _Pragma("unroll") FMM_EACH_EDGE d[u] = sop_eval(K_, d[u], tab); \
+      break;
+         FMM_SOP_CASE(SOP_SIGMOID)
+         FMM_SOP_CASE(SOP_TDIST)
+         FMM_SOP_CASE(SOP_FR)
+         FMM_SOP_CASE(SOP_LL)
+         FMM_SOP_CASE(SOP_FA)
+#undef FMM_SOP_CASE
+         default: break;
+      }
+   }
+   if (vsc == kVscMul)
+   {
+#pragma unroll
+      FMM_EACH_EDGE
+      {
+#pragma unroll
+         for (int r = 0; r < R; r++)
+         {
+            ys[u].v[r].x = d[u] * ys[u].v[r].x; ys[u].v[r].y = d[u] * ys[u].v[r].y;
+            ys[u].v[r].z = d[u] * ys[u].v[r].z; ys[u].v[r].w = d[u] * ys[u].v[r].w;
+         }
+      }
+   }
+   else if (vsc == kVscAdd)
+   {
+#pragma unroll
+      FMM_EACH_EDGE
+      {
+#pragma unroll
+         for (int r = 0; r < R; r++)
+         {
+            ys[u].v[r].x = d[u] + ys[u].v[r].x; ys[u].v[r].y = d[u] + ys[u].v[r].y;
+            ys[u].v[r].z = d[u] + ys[u].v[r].z; ys[u].v[r].w = d[u] + ys[u].v[r].w;
+         }
+      }
+   }
+   if (aop == kAopAdd)
+   {
+#pragma unroll
+      FMM_EACH_EDGE map2(acc, acc, ys[u], [&](real_t a, real_t b) { return ok[u] ? a + b : a; });
+   }
+   else if (aop == kAopMax)
+   {
+#pragma unroll
+      FMM_EACH_EDGE map2(acc, acc, ys[u], [&](real_t a, real_t b) { return ok[u] ? (a > b ? a : b) : a; });
+   }
+   else if (aop == kAopMin)
+   {
+#pragma unroll
+      FMM_EACH_EDGE map2(acc, acc, ys[u], [&](real_t a, real_t b) { return ok[u] ? (a < b ? a : b) : a; });
+   }
+#undef FMM_EACH_EDGE
+}
+
+// A batch in which only the first `nu` (wave-uniform) of the U edges per sub-wave
+// exist, the short last batch of a row, goes through the pipeline at half, a
+// quarter, ... of the width instead of carrying empty edges through every stage.
+template <int L, int R, int U>
+__device__ __forceinline__ void general_group(Slice<R> &acc, const Slice<R> &xs, Slice<R> *ys, const real_t *ev,
+                                              const bool *ok, int nu, int sop_kind, int imsg, const real_t *tab)
+{
+   if constexpr (U >= 2)
+   {
+      if (nu <= U / 2)
+      {
+         general_group<L, R, U / 2>(acc, xs, ys, ev, ok, nu, sop_kind, imsg, tab);
+         return;
+      }
+   }
+   general_steps<L, R, U>(acc, xs, ys, ev, ok, sop_kind, imsg, tab);
+}
+
+// Whole-wave rows take the U edges in flight through the pipeline together.  Sub-waves
+// take them two at a time: all at once would hold every stage's temporaries for all of
+// them in registers and cost a resident workgroup per CU (measured on the K=128 sigmoid
+// and K=64 t-dist benchmarks: 1.69 against 1.86 ms and 24.5 against 25.5 ms; K=256 and
+// K=512 are 3 % and 1 % slower in pairs).
+template <int L, int R, int U>
+__device__ __forceinline__ void general_batch(Slice<R> &acc, const Slice<R> &xs, Slice<R> *ys, const real_t *ev,
+                                              const bool *ok, int nu, int sop_kind, int imsg, const real_t *tab)
+{
+   constexpr int G = ((L == 64 && R <= 2) || U < 2) ? U : 2;   // rows wider than 512 columns: pairs as well
+#pragma unroll
+   for (int g0 = 0; g0 < U; g0 += G)
+      if (g0 < nu) general_group<L, R, G>(acc, xs, ys + g0, ev + g0, ok + g0, nu - g0, sop_kind, imsg, tab);
 }
 
 // 64 consecutive edge slots of a row, one per lane: column id and edge value.
@@ -648,10 +787,26 @@ __device__ __forceinline__ void walk_edges(Slice<R> &acc, const Slice<R> &xs, co
          }
 #pragma unroll
          for (int u = 0; u < U; u++)
+         {
             if (ok[u]) load_slice<V, L, R, EXACT>(ys[u], p.y + (int64_t)col[u] * p.ldy, sl, p.k);
+            else if (OP == OP_GENERIC)
+            {
 #pragma unroll
-         for (int u = 0; u < U; u++)
-            if (ok[u]) edge_step<L, R, OP>(acc, xs, ys[u], ev[u], sop_kind, p.imessage, tab);
+               for (int r = 0; r < R; r++) ys[u].v[r] = zero4();
+            }
+         }
+         if constexpr (OP == OP_GENERIC)
+         {
+            const int in_batch = n - b0;      // > 0; edges e = b0 + u*S + sub of this batch exist for e < n
+            const int nu = in_batch >= S * U ? U : (in_batch + S - 1) / S;
+            general_batch<L, R, U>(acc, xs, ys, ev, ok, nu, sop_kind, p.imessage, tab);
+         }
+         else
+         {
+#pragma unroll
+            for (int u = 0; u < U; u++)
+               if (ok[u]) edge_step<L, R, OP>(acc, xs, ys[u], ev[u], sop_kind, tab);
+         }
       }
       cur = nxt;
       if (left <= 64) break;

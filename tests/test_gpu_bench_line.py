@@ -1,0 +1,44 @@
+"""bench.py end to end on the smallest workload: the JSON line's contract, and the
+variants of the measurement (general pipeline, int64 indices, double precision)."""
+import json
+import os
+import subprocess
+import sys
+
+import pytest
+
+pytestmark = pytest.mark.gpu
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def _bench(*flags):
+    r = subprocess.run([sys.executable, os.path.join(ROOT, "bench.py"), "--workload", "c1", "--steps", "3", "--warmup", "1",
+                        "--no-cpu"] + list(flags), stdout=subprocess.PIPE, stderr=subprocess.PIPE, text=True, timeout=170)
+    assert r.returncode == 0, r.stderr[-2000:]
+    lines = [ln for ln in r.stdout.splitlines() if ln.strip()]
+    assert len(lines) == 1                                    # ONE JSON line
+    return json.loads(lines[0])
+
+
+@pytest.mark.parametrize("flags,pipeline,bits,dtype", [
+    ((), "optimised", 32, "f32"),
+    (("--general",), "general", 32, "f32"),
+    (("--index-bits", "64"), "optimised", 64, "f32"),
+    (("--general", "--index-bits", "64"), "general", 64, "f32"),
+    (("--dtype", "f64"), "optimised", 32, "f64"),
+])
+def test_bench_line(flags, pipeline, bits, dtype):
+    out = _bench(*flags)
+    for key in ("metric", "value", "unit", "n_gpus", "steps", "warmup", "ms_per_step", "higher_is_better", "scaling",
+                "vs_baseline", "dtype", "data", "config", "roofline"):
+        assert key in out, key
+    assert out["n_gpus"] == 1 and out["steps"] == 3 and out["warmup"] == 1 and out["vs_baseline"] is None
+    assert out["dtype"] == dtype and out["config"]["pipeline"] == pipeline and out["config"]["index_bits"] == bits
+    assert out["spot_check_vs_oracle"] is True and out["value"] > 0
+    rl = out["roofline"]
+    assert rl["bound"] == "hbm" and rl["peak"] == 8000.0 and abs(rl["frac"] - rl["achieved"] / rl["peak"]) < 1e-12
+    # c1 is 262 144 edges of 32 columns: 132 bytes per edge and 264 per row with int32 indices and float values
+    vb, ib = (8 if dtype == "f64" else 4), bits // 8
+    want = 262144 * (32 * vb + ib) + 16384 * ((3 if pipeline == "general" else 2) * 32 * vb + 2 * ib)
+    assert rl["algorithmic_bytes"] == want
+    assert rl["traffic"] is None                              # c1 is cache-resident: no counter traffic is quoted for it
