@@ -238,12 +238,19 @@ __device__ __forceinline__ int64_t lane_value<int64_t>(int64_t v, int t)
    return ((int64_t)hi << 32) | (uint32_t)lo;
 }
 
+// The sigmoid table as the fused kernel reads it: always the workgroup's copy in LDS.
+// The pointer carries the address space in its type, so that a look-up is an LDS read
+// (its own counter) also where the SOP body is picked at run time; through a plain
+// pointer it would be a flat load, which waits behind every gather in flight.
+typedef const __attribute__((address_space(3))) real_t *lds_table_t;
+
 // ---- SOP bodies ---------------------------------------------------------------
 // Same expressions, in the same precision, as the SOP_UDEF_FUNC bodies of the
 // reference's tester (test/fusedMMtime.cpp:606-660): constants there are double
 // literals, so the arithmetic is done in double and (single-precision build)
 // rounded once to float.
-__device__ __forceinline__ real_t sop_eval(int kind, real_t s, const real_t *tab)
+template <typename TabPtr>
+__device__ __forceinline__ real_t sop_eval(int kind, real_t s, TabPtr tab)
 {
    switch (kind)
    {
@@ -497,7 +504,7 @@ __device__ __forceinline__ real_t vop_rop(Slice<R> &t, const Slice<R> &xs, const
 // general pipeline is general_steps below.)
 template <int L, int R, int OP>
 __device__ __forceinline__ void edge_step(Slice<R> &acc, const Slice<R> &xs, const Slice<R> &ys,
-                                          real_t edge_val, int sop_kind, const real_t *tab)
+                                          real_t edge_val, int sop_kind, lds_table_t tab)
 {
    static_assert(OP != OP_GENERIC, "the general pipeline goes through general_steps");
    if (OP == OP_GCN)
@@ -538,7 +545,7 @@ __device__ __forceinline__ void edge_step(Slice<R> &acc, const Slice<R> &xs, con
 // with ok[u] false change nothing.  ys[u] is overwritten with T.
 template <int L, int R, int U>
 __device__ __forceinline__ void general_steps(Slice<R> &acc, const Slice<R> &xs, Slice<R> *ys, const real_t *ev,
-                                              const bool *ok, int sop_kind, int imsg, const real_t *tab)
+                                              const bool *ok, int sop_kind, int imsg, lds_table_t tab)
 {
    const int vop = imsg & 0xF, rop = imsg & 0xF0, sop = imsg & 0xF00, vsc = imsg & 0xF000, aop = imsg & 0xF0000;
 #define FMM_EACH_EDGE for (int u = 0; u < U; u++)
@@ -669,7 +676,7 @@ __device__ __forceinline__ void general_steps(Slice<R> &acc, const Slice<R> &xs,
 // quarter, ... of the width instead of carrying empty edges through every stage.
 template <int L, int R, int U>
 __device__ __forceinline__ void general_group(Slice<R> &acc, const Slice<R> &xs, Slice<R> *ys, const real_t *ev,
-                                              const bool *ok, int nu, int sop_kind, int imsg, const real_t *tab)
+                                              const bool *ok, int nu, int sop_kind, int imsg, lds_table_t tab)
 {
    if constexpr (U >= 2)
    {
@@ -689,7 +696,7 @@ __device__ __forceinline__ void general_group(Slice<R> &acc, const Slice<R> &xs,
 // K=512 are 3 % and 1 % slower in pairs).
 template <int L, int R, int U>
 __device__ __forceinline__ void general_batch(Slice<R> &acc, const Slice<R> &xs, Slice<R> *ys, const real_t *ev,
-                                              const bool *ok, int nu, int sop_kind, int imsg, const real_t *tab)
+                                              const bool *ok, int nu, int sop_kind, int imsg, lds_table_t tab)
 {
    constexpr int G = ((L == 64 && R <= 2) || U < 2) ? U : 2;   // rows wider than 512 columns: pairs as well
 #pragma unroll
@@ -751,7 +758,7 @@ __device__ __forceinline__ double chunk_entry(double v, int e)
 template <int V, int L, int R, bool EXACT, int OP, int SOPK, int U, typename IdxT>
 __device__ __forceinline__ void walk_edges(Slice<R> &acc, const Slice<R> &xs, const Params<IdxT> &p,
                                            IdxT jb, IdxT je, EdgeChunk<IdxT> &cur, IdxT next_b, IdxT next_e, int lane,
-                                           const real_t *tab)
+                                           lds_table_t tab)
 {
    constexpr int S = 64 / L;
    const int sub = (L == 64) ? 0 : lane / L, sl = (L == 64) ? lane : lane % L;
@@ -852,12 +859,14 @@ __device__ __forceinline__ bool op_reads_x(int imsg)
    return false;
 }
 
-__device__ __forceinline__ const real_t *stage_table(const real_t *gtab, real_t *lds, bool need)
+__device__ __forceinline__ lds_table_t stage_table(const real_t *gtab, real_t *lds, bool need)
 {
-   if (!need) return gtab;
-   for (int i = threadIdx.x; i < kSigmoidTableSize; i += kBlockThreads) lds[i] = gtab[i];
-   __syncthreads();
-   return lds;
+   if (need)
+   {
+      for (int i = threadIdx.x; i < kSigmoidTableSize; i += kBlockThreads) lds[i] = gtab[i];
+      __syncthreads();
+   }
+   return (lds_table_t)lds;      // read only when `need` held
 }
 
 // Turn the value an atomicAdd on counter `cur` returned (in lane 0) into a
@@ -970,7 +979,7 @@ __global__ __launch_bounds__(kBlockThreads) void classify_kernel(const Params<Id
 
 // ---- phase A of the fused kernel: one wavefront per queued edge segment -> partial Z ----
 template <int V, int L, int R, bool EXACT, int OP, int SOPK, int U, typename IdxT>
-__device__ __forceinline__ void segments_phase(const Params<IdxT> &p, const real_t *tab)
+__device__ __forceinline__ void segments_phase(const Params<IdxT> &p, lds_table_t tab)
 {
    unsigned int nseg = p.ctr->n_seg;
    if (nseg > p.cap_seg) nseg = p.cap_seg;   // rows beyond the cap are done whole in phase B
@@ -1038,7 +1047,7 @@ __device__ __forceinline__ void segments_phase(const Params<IdxT> &p, const real
 
 // ---- phase B of the fused kernel: one wavefront per row ---------------------------
 template <int V, int L, int R, bool EXACT, int OP, int SOPK, int U, typename IdxT>
-__device__ __forceinline__ void rows_phase(const Params<IdxT> &p, const real_t *tab)
+__device__ __forceinline__ void rows_phase(const Params<IdxT> &p, lds_table_t tab)
 {
    const int lane = threadIdx.x & 63;
    const int sub = lane / L, sl = lane % L;
@@ -1235,7 +1244,7 @@ __global__ __launch_bounds__(kBlockThreads) void fused_kernel(const Params<IdxT>
 {
    __shared__ real_t lds_tab[(OP >= OP_DOT) ? kSigmoidTableSize : 1];
    const bool uses_sop = (OP == OP_DOT || OP == OP_DIST || (OP == OP_GENERIC && (p.imessage & 0xF00) == kSopUdef));
-   const real_t *tab = stage_table(p.sigmoid_table, lds_tab, (OP >= OP_DOT) && uses_sop && (SOPK >= 0 ? SOPK : p.sop_kind) == SOP_SIGMOID);
+   const lds_table_t tab = stage_table(p.sigmoid_table, lds_tab, (OP >= OP_DOT) && uses_sop && (SOPK >= 0 ? SOPK : p.sop_kind) == SOP_SIGMOID);
    segments_phase<V, L, R, EXACT, OP, SOPK, U, IdxT>(p, tab);
    rows_phase<V, L, R, EXACT, OP, SOPK, U, IdxT>(p, tab);
    retire_wave<IdxT>(p);
