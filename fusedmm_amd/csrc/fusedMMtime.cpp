@@ -3,7 +3,7 @@
 // :1758-1804) plus a GPU path:
 //
 //   xfusedMMtime_i64 -input graph.mtx -K 128 -t s -T 1 -nrep 20 [-M rows]
-//                    [-C cacheKB] [-skHd 1] [-ibeta 0|1] [-gpu 0|1] [-prof 1]
+//                    [-C cacheKB] [-skHd 1] [-ibeta 0|1] [-gpu 0|1] [-opt 1|0|2] [-prof 1]
 //
 //   -t <t|f|s|m|g>  op kind: t-dist, FR, sigmoid, spmm, gcn.  The reference
 //                   builds one executable per kind (-D<KIND>_UDEF); here one
@@ -19,6 +19,10 @@
 //                   between calls (fusedMM_amd_set_cache), so only C travels.
 //   -C <KB>         rotate through enough operand copies to exceed this cache
 //                   size (reference :1533-1654); default 0 = one copy.
+//   -opt 1          (default) tuples with an optimised kernel use it: the reference's
+//                   xsOptFusedMMtime_* executables (built with ENABLE_OPT_FUSEDMM);
+//   -opt 0          every tuple goes through the general pipeline: its xsFusedMMtime_*;
+//   -opt 2          as 1, and a tuple without an optimised kernel is an error (MUST_OPT_FUSEDMM).
 //   -prof 1         wrap the phases in roctx ranges for rocprofv3 --marker-trace.
 //
 // "Trusted" CPU kernels restate test/fusedMMtime.cpp:159-365; inputs follow
@@ -186,6 +190,8 @@ static void usage()
    printf("-ibeta <1,0>, beta 1.0 or 0.0\n");
    printf("-gpu <0,1>, 1: operands resident on the GPU while timing (default); 0: host pointers\n");
    printf("-cache <0,1>, with -gpu 0: keep device mirrors of the read-only operands between calls\n");
+   printf("-opt <1,0,2>, 1: optimised kernels for the tuples that have one (the reference's xsOptFusedMMtime_*), "
+          "0: general pipeline for every tuple (its xsFusedMMtime_*), 2: as 1, and a tuple without one is an error\n");
    printf("-prof <0,1>, 1: emit roctx ranges\n");
    printf("-h, show this usage message\n");
 }
@@ -194,7 +200,7 @@ int main(int narg, char **argv)
 {
    std::string inputfile;
    IT M = 0, K = 128;
-   int csKB = 0, nrep = 20, isTest = 0, skHd = 0, ibeta = 0, use_gpu_resident = 1, use_cache = 0;
+   int csKB = 0, nrep = 20, isTest = 0, skHd = 0, ibeta = 0, use_gpu_resident = 1, use_cache = 0, opt = 1;
    char tkern = 's';
    const std::string exe = argv[0];
    if (exe.find("_tdist_") != std::string::npos) tkern = 't';
@@ -217,6 +223,7 @@ int main(int narg, char **argv)
       else if (!strcmp(argv[p], "-ibeta")) ibeta = atoi(argv[p + 1]);
       else if (!strcmp(argv[p], "-gpu")) use_gpu_resident = atoi(argv[p + 1]);
       else if (!strcmp(argv[p], "-cache")) use_cache = atoi(argv[p + 1]);
+      else if (!strcmp(argv[p], "-opt")) opt = atoi(argv[p + 1]);
       else if (!strcmp(argv[p], "-prof")) g_prof = atoi(argv[p + 1]) != 0;
    }
    if (inputfile.empty()) { printf("Need input file ??? \n"); return 1; }
@@ -235,6 +242,7 @@ int main(int narg, char **argv)
    assert(N && M && K);
    init_table();
    fusedMM_amd_set_sop_kind(sop_kind_for(tkern));
+   fusedMM_amd_set_opt(opt);
    const int32_t imsg = message_for(tkern);
 
    // inputs as the reference's tester draws them

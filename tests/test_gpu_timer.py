@@ -31,6 +31,20 @@ def test_timer_passes_its_tester(tmp_path, tkern, k, bits):
     assert float(f[6]) > 0 and float(f[8]) > 0
 
 
+@pytest.mark.parametrize("tkern,k", [("s", 128), ("f", 32), ("m", 64)])
+def test_timer_general_pipeline(tmp_path, tkern, k):
+    """-opt 0: what the reference's xsFusedMMtime_* executables (no ENABLE_OPT_FUSEDMM) run,
+    the general pipeline for the same tuples; -opt 2 (MUST_OPT_FUSEDMM) still finds the
+    optimised kernels of these tuples."""
+    g = synth.er_graph(4096, 32768, 5, 32)
+    path = str(tmp_path / "er.mtx")
+    synth.write_mtx_symmetric(path, g)
+    for opt in ("0", "2"):
+        r = subprocess.run([fbuild.timer_path(32), "-input", path, "-T", "1", "-K", str(k), "-t", tkern, "-nrep", "2",
+                            "-opt", opt], stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True, timeout=110)
+        assert r.returncode == 0 and "PASSED TEST" in r.stdout, r.stdout
+
+
 def test_timer_host_pointer_mode(tmp_path):
     g = synth.er_graph(2048, 16384, 2, 64)
     path = str(tmp_path / "er.mtx")
