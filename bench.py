@@ -188,6 +188,9 @@ def main():
                          "timed region samples rather than instruments every step")
     ap.add_argument("--read-probe", action="store_true",
                     help="also time a read-only stream over 4 GiB (what HBM delivers to reads alone) and report it")
+    ap.add_argument("--gather-probe", action="store_true",
+                    help="also time a read-only gather of uniformly random rows of the workload's row size from a buffer "
+                         "the size of its Y (what the memory system delivers to such gathers alone) and report it")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py: this path is built and measured on ONE GPU; --gpus %d is not supported "
@@ -263,6 +266,32 @@ def main():
             read_probe[label + "_GBps"] = nbytes / (e0.elapsed_time(e1) / 10 * 1e-3) / 1e9
         del src, sink
 
+    gather_probe = None
+    row_bytes = k * (vbits // 8)
+    if args.gather_probe and row_bytes <= 2048 and (row_bytes & (row_bytes - 1)) == 0 and row_bytes >= 16:
+        nbytes = n * row_bytes
+        src = torch.empty(nbytes // 4, dtype=torch.float32, device=dev).uniform_(-1, 1)
+        sink = torch.zeros(4, dtype=torch.int32, device=dev)
+        n_ids = (4 << 30) // row_bytes                       # 4 GiB gathered per launch
+        gen = torch.Generator(device=dev)
+        gen.manual_seed(11)
+        ids = torch.randint(0, n, (n_ids,), device=dev, dtype=torch.int64, generator=gen).to(torch.int32)
+        gather_probe = {"row_bytes": row_bytes, "buffer_bytes": nbytes, "gathered_bytes": n_ids * row_bytes}
+        for label, nt in (("plain_loads", 0), ("nontemporal_loads", 1)):
+            launch = lambda: lib.fusedMM_amd_gather_probe(src.data_ptr(), row_bytes, ids.data_ptr(), n_ids, 4, 8, nt,
+                                                          sink.data_ptr(), stream)
+            for _ in range(2):
+                assert launch() == 0
+            torch.cuda.synchronize()
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record()
+            for _ in range(10):
+                launch()
+            e1.record()
+            torch.cuda.synchronize()
+            gather_probe[label + "_GBps"] = n_ids * row_bytes / (e0.elapsed_time(e1) / 10 * 1e-3) / 1e9
+        del src, sink, ids
+
     for _ in range(args.warmup):
         step()
     torch.cuda.synchronize()
@@ -308,6 +337,10 @@ def main():
     if read_probe:
         roofline["read_stream_probe"] = read_probe
         roofline["frac_of_read_stream"] = achieved / read_probe["plain_loads_GBps"]
+
+    if gather_probe:
+        roofline["gather_probe"] = gather_probe
+        roofline["frac_of_gather_probe"] = achieved / gather_probe["plain_loads_GBps"]
 
     checked = None
     if not args.no_check:

@@ -1613,6 +1613,36 @@ int fusedMM_amd_read_probe(const void *src, int64_t bytes, int blocks_per_cu, in
    return hip_status(hipGetLastError(), "read probe launch");
 }
 
+int fusedMM_amd_gather_probe(const void *src, int row_bytes, const unsigned int *ids, int64_t n_ids, int blocks_per_cu,
+                             int in_flight, int nontemporal, void *sink, void *stream)
+{
+   if (!src || !ids || !sink || n_ids < 1 || !aligned16(src)) return FUSEDMM_FAIL_RETURN;
+   if (row_bytes < 16 || row_bytes > 2048 || (row_bytes & (row_bytes - 1))) return FUSEDMM_FAIL_RETURN;
+   std::lock_guard<std::mutex> lock(g.mu);
+   DeviceState *d = nullptr;
+   int st = device_basics(&d);
+   if (st) return st;
+   if (blocks_per_cu < 1) blocks_per_cu = 4;
+   const dim3 grid((unsigned int)(d->num_cu * blocks_per_cu)), block(kBlockThreads);
+   const probe16_t *s4 = (const probe16_t *)src;
+   unsigned int *out = (unsigned int *)sink;
+   const int row16 = row_bytes / 16;
+   hipStream_t hs = (hipStream_t)stream;
+#define FMM_GPROBE(U_, R_)                                                                                              \
+   if (nontemporal) hipLaunchKernelGGL((gather_probe_kernel<U_, R_, true>), grid, block, 0, hs, s4, row16, ids, n_ids, out); \
+   else hipLaunchKernelGGL((gather_probe_kernel<U_, R_, false>), grid, block, 0, hs, s4, row16, ids, n_ids, out)
+   if (row16 > 64)   // 2 KiB rows: two pieces per lane
+   {
+      if (in_flight >= 8) { FMM_GPROBE(8, 2); }
+      else { FMM_GPROBE(4, 2); }
+   }
+   else if (in_flight >= 16) { FMM_GPROBE(16, 1); }
+   else if (in_flight >= 8) { FMM_GPROBE(8, 1); }
+   else { FMM_GPROBE(4, 1); }
+#undef FMM_GPROBE
+   return hip_status(hipGetLastError(), "gather probe launch");
+}
+
 void fusedMM_amd_finalize(void)
 {
    std::lock_guard<std::mutex> lock(g.mu);

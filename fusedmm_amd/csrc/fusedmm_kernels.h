@@ -1445,4 +1445,46 @@ __global__ __launch_bounds__(kBlockThreads) void read_probe_kernel(const probe16
    if (acc == 0x9E3779B9u) *sink = acc;
 }
 
+// Read-only gather of whole rows: row ids[j] of `row16` 16-byte pieces each (a power of
+// two up to 64 * R), for j < n_ids, in the order given; a wavefront takes 64 / L rows at
+// a time on L = min(64, row16) lanes each and keeps U such steps in flight.  Nothing but
+// the loads and an exclusive-or: the yardstick for what the memory system delivers to
+// gathers of rows of this size, as read_probe_kernel is for a stream.
+template <int U, int R, bool NT>
+__global__ __launch_bounds__(kBlockThreads) void gather_probe_kernel(const probe16_t *src, int row16, const unsigned int *ids,
+                                                                     int64_t n_ids, unsigned int *sink)
+{
+   const int lane = threadIdx.x & 63;
+   const int L = row16 / R, S = 64 / L;
+   const int sub = lane / L, sl = lane % L;
+   const int64_t wave = ((int64_t)blockIdx.x * kBlockThreads + threadIdx.x) >> 6;
+   const int64_t nwaves = (int64_t)gridDim.x * (kBlockThreads / 64);
+   unsigned int acc = 0u;
+   for (int64_t b = wave * S * U; b < n_ids; b += nwaves * S * U)
+   {
+      int64_t row[U];
+#pragma unroll
+      for (int u = 0; u < U; u++)
+      {
+         const int64_t j = b + u * S + sub;
+         row[u] = j < n_ids ? (int64_t)ids[j] : -1;
+      }
+      probe16_t v[U][R];
+#pragma unroll
+      for (int u = 0; u < U; u++)
+#pragma unroll
+         for (int r = 0; r < R; r++)
+         {
+            const probe16_t *at = src + row[u] * row16 + r * L + sl;
+            if (row[u] >= 0) v[u][r] = NT ? __builtin_nontemporal_load(at) : *at;
+            else v[u][r] = probe16_t{0u, 0u, 0u, 0u};
+         }
+#pragma unroll
+      for (int u = 0; u < U; u++)
+#pragma unroll
+         for (int r = 0; r < R; r++) acc ^= v[u][r].x ^ v[u][r].y ^ v[u][r].z ^ v[u][r].w;
+   }
+   if (acc == 0x9E3779B9u) *sink = acc;
+}
+
 }  // namespace fmm

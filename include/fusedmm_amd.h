@@ -214,6 +214,17 @@ int fusedMM_amd_copy_probe(void *dst, const void *src, int64_t bytes, void *stre
 int fusedMM_amd_read_probe(const void *src, int64_t bytes, int blocks_per_cu, int in_flight, int nontemporal,
                            void *sink, void *stream);
 
+/* Gather `n_ids` whole rows of `row_bytes` bytes (a power of two, 16..2048) from
+ * `src` at the row numbers ids[0..n_ids) (device memory; the caller keeps them
+ * inside `src`), in that order, with blocks_per_cu workgroups per compute unit
+ * and `in_flight` (4, 8 or 16; 4 or 8 for 2048-byte rows) rows outstanding per
+ * group of lanes that shares a row; nothing else is computed and nothing is
+ * written.  A measuring aid: what the memory system delivers to gathers of rows
+ * of the size a benchmark gathers, where fusedMM_amd_read_probe gives the rate of
+ * a plain stream. */
+int fusedMM_amd_gather_probe(const void *src, int row_bytes, const unsigned int *ids, int64_t n_ids, int blocks_per_cu,
+                             int in_flight, int nontemporal, void *sink, void *stream);
+
 /* Release every device buffer the library holds (work queues, staging). */
 void fusedMM_amd_finalize(void);
 

@@ -462,3 +462,35 @@ def test_two_host_threads_calling_at_once(oracle):
     for i in range(len(dY)):
         for rep in range(20):
             assert torch.equal(got[i][rep], want[i]), (i, rep)
+
+
+def test_probes_take_what_they_document(oracle):
+    """The measuring aids (copy, read-stream and gather probes) run on well-formed
+    arguments and refuse the rest without launching anything."""
+    import torch
+    lib = fa.load(32)
+    dev = torch.device("cuda:0")
+    st = torch.cuda.current_stream().cuda_stream
+    src = torch.arange(1 << 20, dtype=torch.float32, device=dev)            # 4 MiB
+    dst = torch.zeros_like(src)
+    sink = torch.zeros(4, dtype=torch.int32, device=dev)
+    assert lib.fusedMM_amd_copy_probe(dst.data_ptr(), src.data_ptr(), src.numel() * 4, st) == 0
+    torch.cuda.synchronize()
+    assert torch.equal(dst, src)
+    assert lib.fusedMM_amd_copy_probe(dst.data_ptr(), src.data_ptr(), 24, st) == fa.FAIL           # not a multiple of 16
+    for nt in (0, 1):
+        assert lib.fusedMM_amd_read_probe(src.data_ptr(), src.numel() * 4, 4, 8, nt, sink.data_ptr(), st) == 0
+    assert lib.fusedMM_amd_read_probe(src.data_ptr() + 4, 1024, 4, 8, 0, sink.data_ptr(), st) == fa.FAIL   # misaligned
+    for row_bytes in (16, 128, 256, 1024, 2048):
+        rows = src.numel() * 4 // row_bytes
+        ids = torch.randint(0, rows, (5000,), device=dev, dtype=torch.int64).to(torch.int32)
+        for nt in (0, 1):
+            for in_flight in (4, 8, 16):
+                assert lib.fusedMM_amd_gather_probe(src.data_ptr(), row_bytes, ids.data_ptr(), ids.numel(), 2, in_flight, nt,
+                                                    sink.data_ptr(), st) == 0
+    ids = torch.zeros(8, dtype=torch.int32, device=dev)
+    for bad in (0, 8, 48, 4096):
+        assert lib.fusedMM_amd_gather_probe(src.data_ptr(), bad, ids.data_ptr(), 8, 2, 8, 0, sink.data_ptr(), st) == fa.FAIL
+    assert lib.fusedMM_amd_gather_probe(src.data_ptr(), 256, ids.data_ptr(), 0, 2, 8, 0, sink.data_ptr(), st) == fa.FAIL
+    torch.cuda.synchronize()
+    assert int(sink.abs().sum()) == 0                                       # the probes store nothing
