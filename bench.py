@@ -51,6 +51,11 @@ WORKLOADS = {
     "c4g": ("gcn K=64 on the c4 graph (same gathers, no reduction or scalar op)", "g", 64, None),
     "c5": ("sigmoid K=512, Zipf(1.8) degrees n=2^21 nnz~4e7, hubs to 1e6", "s", 512, "sigmoid"),
 }
+# What a row length costs: sigmoid K=512 over a Y of 2^21 rows (c5's), every row with the
+# same number of uniformly random neighbours, min(2^21, 2^25 / degree) rows.
+for _d in (1, 4, 16, 64, 512):
+    WORKLOADS["u512d%d" % _d] = ("sigmoid K=512, %d rows of %d uniform neighbours each among 2^21" % (
+        min(1 << 21, (1 << 25) // _d), _d), "s", 512, "sigmoid")
 
 
 def make_workload(name, scale_down=0):
@@ -79,6 +84,12 @@ def make_workload(name, scale_down=0):
         n = (1 << 21) >> sd
         g = synth.zipf_graph(n, 1.8, min(1000000, n // 2), 40000000 >> sd, 5)
         return g, synth.uniform_matrix(n, 512, -0.5, 0.5, 5, 1), synth.uniform_matrix(n, 512, -0.5, 0.5, 5, 2)
+    if name.startswith("u512d"):
+        d = int(name[5:])
+        n = (1 << 21) >> sd
+        m = min(n, ((1 << 25) >> sd) // d)
+        g = synth.uniform_degree_graph(n, m, d, 6)
+        return g, synth.uniform_matrix(m, 512, -0.5, 0.5, 6, 1), synth.uniform_matrix(n, 512, -0.5, 0.5, 6, 2)
     raise SystemExit("unknown workload %s" % name)
 
 
@@ -170,7 +181,9 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=3)
-    ap.add_argument("--workload", default="c2", choices=sorted(WORKLOADS))
+    ap.add_argument("--workload", default="c2", choices=sorted(WORKLOADS),
+                    help="c1-c5: the benchmark configurations (c2 is the one the metric is quoted on); c3g, c4g: the gcn "
+                         "tuple on the c3 and c4 graphs; u512d<D>: uniform-degree rows at c5's row size (a measuring aid)")
     ap.add_argument("--dtype", default="f32", choices=["f32", "f64"],
                     help="f64 runs the double-precision library (the reference's -DDREAL build)")
     ap.add_argument("--index-bits", type=int, default=32, choices=[32, 64],

@@ -127,6 +127,16 @@ def zipf_graph(n, exponent, cap, target_nnz, seed, index_bits=32, n_hubs=4):
     return _csr_from_keys(n, keys, index_bits)
 
 
+def uniform_degree_graph(n, m, degree, seed, index_bits=32):
+    """m rows of exactly `degree` uniformly random neighbours among n columns
+    (unsorted, repeats possible): every row costs the same, so what a row
+    length costs can be read off a run."""
+    rng = _rng(seed)
+    indx = rng.integers(0, n, m * degree, dtype=np.int64)
+    rowptr = np.arange(m + 1, dtype=np.int64) * degree
+    return graph_from_rowptr(m, n, rowptr, indx, None, index_bits)
+
+
 def uniform_matrix(n, k, lo, hi, seed, stream=1):
     rng = _rng(seed, stream)
     out = rng.random((n, k), dtype=np.float32)
