@@ -4,9 +4,10 @@
 // row).  A wavefront is cut into S = 64/L sub-waves of L lanes; a sub-wave owns
 // one neighbour row Y[c] at a time, each lane holding R four-element slices of
 // it, so a gather is L coalesced 16-byte loads (two per lane in double
-// precision).  The X[i] slice and the Z accumulator live in VGPRs for the whole row.  The per-edge reduction (ROP) is a DPP /
-// swizzle XOR butterfly over the L lanes, the scalar op (SOP) and the scaled
-// accumulate (MOP, AOP) happen in registers.
+// precision).  The X[i] slice and the Z accumulator live in VGPRs for the whole
+// row.  The per-edge reduction (ROP) is a DPP / swizzle XOR butterfly over the L
+// lanes, the scalar op (SOP) and the scaled accumulate (MOP, AOP) happen in
+// registers.
 //
 // Element e of a K-vector sits in lane (e/4) % L, register (e/4) / L,
 // component e % 4.  A lane reduces its own elements with a fused multiply-add
