@@ -259,24 +259,25 @@ __device__ __forceinline__ real_t sop_eval(int kind, real_t s, TabPtr tab)
       {
          // floor-indexed 2048-entry table on [-5,5] (test/fusedMMtime.cpp:128-130, 606-611);
          // s == 5 exactly would index one past the end there: clamp to the last entry.
-         real_t t;
-         if (s > (real_t)5.0) t = (real_t)1.0;
-         else if (s < (real_t)-5.0) t = (real_t)0.0;
-         else
-         {
+         // Written without branches (the look-up is made for every lane, from a clamped
+         // argument, and the saturated ends are selected afterwards): lanes of a wave
+         // take different sides, and straight-line code lets the look-ups of the edges
+         // in flight overlap.
+         const real_t sc = s > (real_t)5.0 ? (real_t)5.0 : (s < (real_t)-5.0 ? (real_t)-5.0 : s);
 #ifdef FMM_DOUBLE
-            int idx = (int)((s + 5.0) * 2048.0 / 10.0);
+         int idx = (int)((sc + 5.0) * 2048.0 / 10.0);
 #else
-            // The reference evaluates ((double)s + 5.0) * 2048 / 10.0.  One multiply by
-            // 204.8 truncates to the same integer for every float in [-5, 5]
-            // (checked exhaustively over all 2 168 455 170 of them on the CPU), and
-            // spares a double-precision division per edge.
-            int idx = (int)(((double)s + 5.0) * 204.8);
+         // The reference evaluates ((double)s + 5.0) * 2048 / 10.0.  One multiply by
+         // 204.8 truncates to the same integer for every float in [-5, 5]
+         // (checked exhaustively over all 2 168 455 170 of them on the CPU), and
+         // spares a double-precision division per edge.
+         int idx = (int)(((double)sc + 5.0) * 204.8);
 #endif
-            idx = idx > kSigmoidTableSize - 1 ? kSigmoidTableSize - 1 : idx;
-            idx = idx < 0 ? 0 : idx;   // only a NaN gets here (neither comparison above holds for it)
-            t = tab[idx];
-         }
+         idx = idx > kSigmoidTableSize - 1 ? kSigmoidTableSize - 1 : idx;
+         idx = idx < 0 ? 0 : idx;   // only a NaN gets here (no comparison holds for it)
+         real_t t = tab[idx];
+         t = s > (real_t)5.0 ? (real_t)1.0 : t;
+         t = s < (real_t)-5.0 ? (real_t)0.0 : t;
          return (real_t)1.0 - t;   // single precision: exact in double for table values, one rounding either way
       }
       case SOP_TDIST:
