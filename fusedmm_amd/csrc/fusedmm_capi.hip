@@ -88,6 +88,7 @@ struct DeviceState {
    Counters *ctr = nullptr;
    Buffer heavy, segs, partial, queued;
    Buffer stage[8];           // host-pointer mode: pntrb, pntre, indx, val, x, y, z, spare
+   Buffer edge_t;             // per-edge vectors T[j][0..k) of the stage-by-stage path (host-function stages)
    // host-pointer mode: two pinned buffers each way, copies are pipelined through them
    void *pin[4] = {nullptr, nullptr, nullptr, nullptr};
    hipEvent_t pin_ev[4];
@@ -125,6 +126,10 @@ struct Globals {
    double phase_ms[3] = {0, 0, 0};   // upload, kernels, download of the last host-pointer call
    bool phase_valid = false;
    fusedMM_amd_sop_fn sop_fn = nullptr;
+   fusedMM_amd_vop_fn vop_fn = nullptr;
+   fusedMM_amd_rop_fn rop_fn = nullptr;
+   fusedMM_amd_vsc_fn vsc_fn = nullptr;
+   fusedMM_amd_aop_fn aop_fn = nullptr;
    int timing = 0;            // 0: off; n: HIP events around the kernels of every n-th call
    int timing_seen = 0;       // calls since timing was switched on
    int timing_calls = 0;      // calls recorded
@@ -386,7 +391,9 @@ struct Plan {
    bool opt_rule;     // optimised write-back rule (beta == 0 overwrites)
    bool needs_sop;    // tuple uses SOP_UDEF
    bool reads_x, reads_val;
+   int udef_stages;   // stages that are the caller's host functions: kUdefVop | kUdefRop | kUdefVsc | kUdefAop
 };
+enum : int { kUdefVop = 1, kUdefRop = 2, kUdefVsc = 4, kUdefAop = 8 };
 
 // Stage validation in the order of reference fusedMM.c:610-628, then the
 // pattern match of :523-583.
@@ -395,15 +402,17 @@ int make_plan(int32_t imsg, int opt_enabled, Plan *pl)
    const int vop = GET_VOP_FLAG(imsg), rop = GET_ROP_FLAG(imsg), sop = GET_SOP_FLAG(imsg),
              vsc = GET_VSC_FLAG(imsg), aop = GET_AOP_FLAG(imsg);
    if (imsg & ~0xFFFFF) { FMM_LOG("Unknown bits in imessage 0x%x", imsg); return FUSEDMM_FAIL_RETURN; }
-   if (vop == VOP_UDEF) { FMM_LOG("VOP_UDEF has no device implementation"); return FUSEDMM_UNDEFINED_USER_FUNCTION; }
-   if (vop < VOP_COPY_LHS || vop > VOP_MIN) { FMM_LOG("Unknown VOP Message"); return FUSEDMM_VOP_FAIL_RETURN; }
-   if (rop == ROP_UDEF) { FMM_LOG("ROP_UDEF has no device implementation"); return FUSEDMM_UNDEFINED_USER_FUNCTION; }
-   if (rop > ROP_NORMR) { FMM_LOG("Unknown ROP Message"); return FUSEDMM_ROP_FAIL_RETURN; }
+   // A *_UDEF stage is the caller's host function (the entry point checks that there is one).
+   pl->udef_stages = 0;
+   if (vop == VOP_UDEF) pl->udef_stages |= kUdefVop;
+   else if (vop < VOP_COPY_LHS || vop > VOP_MIN) { FMM_LOG("Unknown VOP Message"); return FUSEDMM_VOP_FAIL_RETURN; }
+   if (rop == ROP_UDEF) pl->udef_stages |= kUdefRop;
+   else if (rop > ROP_NORMR) { FMM_LOG("Unknown ROP Message"); return FUSEDMM_ROP_FAIL_RETURN; }
    if (!(sop == SOP_NOOP || sop == SOP_COPY || sop == SOP_UDEF)) { FMM_LOG("Unknown SOP Message"); return FUSEDMM_SOP_FAIL_RETURN; }
-   if (vsc == VSC_UDEF) { FMM_LOG("VSC_UDEF has no device implementation"); return FUSEDMM_UNDEFINED_USER_FUNCTION; }
-   if (vsc > VSC_ADD) { FMM_LOG("Unknown VSC Message"); return FUSEDMM_VSC_FAIL_RETURN; }
-   if (aop == AOP_UDEF) { FMM_LOG("AOP_UDEF has no device implementation"); return FUSEDMM_UNDEFINED_USER_FUNCTION; }
-   if (aop > AOP_MIN) { FMM_LOG("Unknown AOP Message"); return FUSEDMM_AOP_FAIL_RETURN; }
+   if (vsc == VSC_UDEF) pl->udef_stages |= kUdefVsc;
+   else if (vsc > VSC_ADD) { FMM_LOG("Unknown VSC Message"); return FUSEDMM_VSC_FAIL_RETURN; }
+   if (aop == AOP_UDEF) pl->udef_stages |= kUdefAop;
+   else if (aop > AOP_MIN) { FMM_LOG("Unknown AOP Message"); return FUSEDMM_AOP_FAIL_RETURN; }
 
    pl->needs_sop = (sop == SOP_UDEF);
    pl->opt_rule = false;
@@ -427,6 +436,12 @@ int make_plan(int32_t imsg, int opt_enabled, Plan *pl)
                  (pl->op == OP_GENERIC && (vop != VOP_COPY_RHS || rop == ROP_DOT || rop == ROP_ADD_LHS || rop == ROP_NORML));
    // the general pipeline seeds the scalar with val[j]; it matters only when no ROP overwrites it
    pl->reads_val = (pl->op == OP_SPMM) || (pl->op == OP_GENERIC && rop == ROP_NOOP && vsc != VSC_NOOP);
+   if (pl->udef_stages)
+   {
+      // a host VOP or ROP is handed X[i]; a host ROP is handed the edge value as the scalar's start
+      if (pl->udef_stages & (kUdefVop | kUdefRop)) pl->reads_x = true;
+      pl->reads_val = (rop == ROP_NOOP && vsc != VSC_NOOP) || rop == ROP_UDEF;
+   }
    return FUSEDMM_SUCCESS_RETURN;
 }
 
@@ -1246,6 +1261,242 @@ int run_host_sop(const Args &a, const idx_t *h_pb, const idx_t *h_pe, int64_t sl
    return hip_status(hipStreamSynchronize(0), "hipStreamSynchronize");
 }
 
+// ---- VOP / ROP / VSC / AOP evaluated by the caller's host functions ---------------------------
+// The reference calls the five stage functions once per edge (fusedMM.c:696-740):
+//    VOP(k, X[i], k, Y[c], k, T); ROP(k, X[i], k, T, &scal); SOP(scal, &out); VSC(k, T, out, k, T); AOP(k, T, k, Z[i])
+// with scal starting as the edge value.  Here T and the scalar of every edge slot live
+// in device buffers; a built-in stage is a kernel over them, a *_UDEF stage is a host
+// pass (the buffers are copied to the host, the caller's function is applied edge by
+// edge -- rows dealt to a few threads, the accumulate stage in edge order within a row
+// -- and copied back), so any mix of built-in and user stages is served and only the
+// user's functions run on the CPU.  Synchronous; device operands `a`, host copies of
+// the row pointers in h_pb / h_pe.
+struct StageFns {
+   fusedMM_amd_vop_fn vop;
+   fusedMM_amd_rop_fn rop;
+   fusedMM_amd_sop_fn sop;
+   fusedMM_amd_vsc_fn vsc;
+   fusedMM_amd_aop_fn aop;
+};
+
+template <class F>
+void for_row_ranges(int64_t m, F body)
+{
+   unsigned int nthreads = std::thread::hardware_concurrency();
+   if (nthreads < 1) nthreads = 1;
+   if (nthreads > 16) nthreads = 16;
+   if ((int64_t)nthreads > m) nthreads = (unsigned int)(m > 0 ? m : 1);
+   std::vector<std::thread> pool;
+   for (unsigned int t = 0; t < nthreads; t++)
+      pool.emplace_back([&, t]() { body(m * t / nthreads, m * (t + 1) / nthreads); });
+   for (auto &th : pool) th.join();
+}
+
+int run_host_stages(const Args &a, const idx_t *h_pb, const idx_t *h_pe, int64_t slots, const Plan &pl, const StageFns &f,
+                    int sop_kind)
+{
+   if (a.m <= 0 || a.k < 1) return FUSEDMM_SUCCESS_RETURN;
+   DeviceState *d = nullptr;
+   int st = device_state(&d);
+   if (st) return st;
+   if (a.ldy < a.k || a.ldz < a.k || (pl.reads_x && a.ldx < a.k))
+   {
+      FMM_LOG("leading dimension smaller than k");
+      return FUSEDMM_FAIL_RETURN;
+   }
+   if (!a.indx || !a.pntrb || !a.pntre || !a.y || !a.z || (pl.reads_x && !a.x))
+   {
+      FMM_LOG("NULL operand");
+      return FUSEDMM_FAIL_RETURN;
+   }
+   if (g.validate)
+   {
+      st = validate_host_pointers_of(a, h_pb, h_pe);
+      if (st) return st;
+      st = validate_operands(a, 0);
+      if (st) return st;
+   }
+   if (slots <= 0) return FUSEDMM_SUCCESS_RETURN;   // no processed row has an edge: Z is left alone (general rule)
+   const int vop = GET_VOP_FLAG(a.imessage), rop = GET_ROP_FLAG(a.imessage), sop = GET_SOP_FLAG(a.imessage),
+             vsc = GET_VSC_FLAG(a.imessage), aop = GET_AOP_FLAG(a.imessage);
+   if ((pl.udef_stages & kUdefVop) && a.n <= 0)
+   {
+      FMM_LOG("VOP_UDEF: n must be the number of rows of Y (the host function is handed rows of a host copy of Y)");
+      return FUSEDMM_FAIL_RETURN;
+   }
+   const int64_t m = a.m, k = a.k;
+   const size_t nT = (size_t)slots * (size_t)k;
+   st = grow(d->edge_t, nT * kValBytes); if (st) return st;
+   st = grow(d->stage[7], (size_t)slots * kValBytes); if (st) return st;
+   val_t *d_T = (val_t *)d->edge_t.ptr, *d_s = (val_t *)d->stage[7].ptr;
+
+   Params<idx_t> p;
+   memset(&p, 0, sizeof(p));
+   p.pntrb = a.pntrb; p.pntre = a.pntre; p.indx = a.indx; p.val = a.val;
+   p.x = a.x ? a.x : a.y;   // built-in stages that never read X still index it; any valid row will do
+   p.y = a.y; p.z = a.z; p.m = m; p.ldx = a.x ? a.ldx : 0; p.ldy = a.ldy; p.ldz = a.ldz; p.k = (int)k;
+   p.imessage = a.imessage;
+   int64_t blocks = (m + kWavesPerBlock - 1) / kWavesPerBlock;
+   if (blocks > (int64_t)d->num_cu * 8) blocks = (int64_t)d->num_cu * 8;
+   const dim3 grid((unsigned int)blocks), block(kBlockThreads);
+
+   // host copies, made when a host stage first needs them
+   std::vector<val_t> hT, hs, hX, hY, hZ;
+   std::vector<idx_t> hidx;
+   bool T_dev = false, T_host = false, s_dev = false, s_host = false;
+   auto need_T_host = [&]() -> int {
+      if (T_host) return FUSEDMM_SUCCESS_RETURN;
+      hT.resize(nT);
+      if (T_dev) FMM_HIP(hipMemcpy(hT.data(), d_T, nT * kValBytes, hipMemcpyDeviceToHost));
+      T_host = true;
+      return FUSEDMM_SUCCESS_RETURN;
+   };
+   auto need_T_dev = [&]() -> int {
+      if (T_dev) return FUSEDMM_SUCCESS_RETURN;
+      if (T_host) FMM_HIP(hipMemcpy(d_T, hT.data(), nT * kValBytes, hipMemcpyHostToDevice));
+      T_dev = true;
+      return FUSEDMM_SUCCESS_RETURN;
+   };
+   auto need_s_host = [&]() -> int {
+      if (s_host) return FUSEDMM_SUCCESS_RETURN;
+      hs.resize((size_t)slots);
+      if (s_dev) FMM_HIP(hipMemcpy(hs.data(), d_s, (size_t)slots * kValBytes, hipMemcpyDeviceToHost));
+      s_host = true;
+      return FUSEDMM_SUCCESS_RETURN;
+   };
+   auto need_s_dev = [&]() -> int {
+      if (s_dev) return FUSEDMM_SUCCESS_RETURN;
+      if (s_host) FMM_HIP(hipMemcpy(d_s, hs.data(), (size_t)slots * kValBytes, hipMemcpyHostToDevice));
+      s_dev = true;
+      return FUSEDMM_SUCCESS_RETURN;
+   };
+   auto need_X_host = [&]() -> int {
+      if (!hX.empty()) return FUSEDMM_SUCCESS_RETURN;
+      hX.resize((size_t)(m - 1) * (size_t)a.ldx + (size_t)k);
+      FMM_HIP(hipMemcpy(hX.data(), a.x, hX.size() * kValBytes, hipMemcpyDeviceToHost));
+      return FUSEDMM_SUCCESS_RETURN;
+   };
+
+   // ---- VOP
+   if (pl.udef_stages & kUdefVop)
+   {
+      st = need_X_host(); if (st) return st;
+      hY.resize((size_t)(a.n - 1) * (size_t)a.ldy + (size_t)k);
+      FMM_HIP(hipMemcpy(hY.data(), a.y, hY.size() * kValBytes, hipMemcpyDeviceToHost));
+      hidx.resize((size_t)slots);
+      FMM_HIP(hipMemcpy(hidx.data(), a.indx, (size_t)slots * sizeof(idx_t), hipMemcpyDeviceToHost));
+      hT.assign(nT, (val_t)0);
+      for_row_ranges(m, [&](int64_t lo, int64_t hi) {
+         for (int64_t i = lo; i < hi; i++)
+            for (int64_t j = (int64_t)h_pb[i]; j < (int64_t)h_pe[i]; j++)
+               (void)f.vop((idx_t)k, hX.data() + i * a.ldx, (idx_t)k, hY.data() + (int64_t)hidx[(size_t)j] * a.ldy, (idx_t)k,
+                           hT.data() + (size_t)j * (size_t)k);
+      });
+      T_host = true;
+   }
+   else
+   {
+      hipLaunchKernelGGL(stage_vop_kernel<idx_t>, grid, block, 0, 0, p, d_T);
+      st = hip_status(hipGetLastError(), "stage kernel launch"); if (st) return st;
+      T_dev = true;
+   }
+
+   // ---- ROP: the scalar starts as the edge value (fusedMM.c:717)
+   if (a.val) FMM_HIP(hipMemcpyAsync(d_s, a.val, (size_t)slots * kValBytes, hipMemcpyDeviceToDevice, 0));
+   else FMM_HIP(hipMemsetAsync(d_s, 0, (size_t)slots * kValBytes, 0));
+   s_dev = true;
+   if (pl.udef_stages & kUdefRop)
+   {
+      st = need_X_host(); if (st) return st;
+      st = need_T_host(); if (st) return st;
+      st = need_s_host(); if (st) return st;
+      for_row_ranges(m, [&](int64_t lo, int64_t hi) {
+         for (int64_t i = lo; i < hi; i++)
+            for (int64_t j = (int64_t)h_pb[i]; j < (int64_t)h_pe[i]; j++)
+               (void)f.rop((idx_t)k, hX.data() + i * a.ldx, (idx_t)k, hT.data() + (size_t)j * (size_t)k, &hs[(size_t)j]);
+      });
+      s_dev = false;
+   }
+   else if (rop != ROP_NOOP)
+   {
+      st = need_T_dev(); if (st) return st;
+      hipLaunchKernelGGL(stage_rop_kernel<idx_t>, grid, block, 0, 0, p, (const val_t *)d_T, d_s);
+      st = hip_status(hipGetLastError(), "stage kernel launch"); if (st) return st;
+   }
+
+   // ---- SOP
+   if (sop == SOP_UDEF && vsc != VSC_NOOP)
+   {
+      if (sop_kind == FUSEDMM_SOP_KIND_HOST)
+      {
+         st = need_s_host(); if (st) return st;
+         for_row_ranges(m, [&](int64_t lo, int64_t hi) {
+            for (int64_t i = lo; i < hi; i++)
+               for (int64_t j = (int64_t)h_pb[i]; j < (int64_t)h_pe[i]; j++)
+               {
+                  val_t out = hs[(size_t)j];
+                  (void)f.sop(hs[(size_t)j], &out);
+                  hs[(size_t)j] = out;
+               }
+         });
+         s_dev = false;
+      }
+      else
+      {
+         st = need_s_dev(); if (st) return st;
+         hipLaunchKernelGGL(apply_sop_kernel, dim3((unsigned int)(d->num_cu * 4)), block, 0, 0, d_s, slots, sop_kind,
+                            (const val_t *)d->sigmoid_table);
+         st = hip_status(hipGetLastError(), "apply sop launch"); if (st) return st;
+         s_host = false;
+      }
+   }
+
+   // ---- VSC
+   if (pl.udef_stages & kUdefVsc)
+   {
+      st = need_T_host(); if (st) return st;
+      st = need_s_host(); if (st) return st;
+      for_row_ranges(m, [&](int64_t lo, int64_t hi) {
+         for (int64_t i = lo; i < hi; i++)
+            for (int64_t j = (int64_t)h_pb[i]; j < (int64_t)h_pe[i]; j++)
+            {
+               val_t *t = hT.data() + (size_t)j * (size_t)k;
+               (void)f.vsc((idx_t)k, t, hs[(size_t)j], (idx_t)k, t);
+            }
+      });
+      T_dev = false;
+   }
+   else if (vsc != VSC_NOOP)
+   {
+      st = need_T_dev(); if (st) return st;
+      st = need_s_dev(); if (st) return st;
+      hipLaunchKernelGGL(stage_vsc_kernel<idx_t>, grid, block, 0, 0, p, d_T, (const val_t *)d_s);
+      st = hip_status(hipGetLastError(), "stage kernel launch"); if (st) return st;
+      T_host = false;
+   }
+
+   // ---- AOP
+   if (pl.udef_stages & kUdefAop)
+   {
+      st = need_T_host(); if (st) return st;
+      hZ.resize((size_t)(m - 1) * (size_t)a.ldz + (size_t)k);
+      FMM_HIP(hipMemcpy(hZ.data(), a.z, hZ.size() * kValBytes, hipMemcpyDeviceToHost));
+      for_row_ranges(m, [&](int64_t lo, int64_t hi) {
+         for (int64_t i = lo; i < hi; i++)
+            for (int64_t j = (int64_t)h_pb[i]; j < (int64_t)h_pe[i]; j++)   // in edge order: the function folds into Z[i]
+               (void)f.aop((idx_t)k, hT.data() + (size_t)j * (size_t)k, (idx_t)k, hZ.data() + i * a.ldz);
+      });
+      FMM_HIP(hipMemcpy(a.z, hZ.data(), hZ.size() * kValBytes, hipMemcpyHostToDevice));
+   }
+   else if (aop != AOP_NOOP)
+   {
+      st = need_T_dev(); if (st) return st;
+      hipLaunchKernelGGL(stage_aop_kernel<idx_t>, grid, block, 0, 0, p, (const val_t *)d_T);
+      st = hip_status(hipGetLastError(), "stage kernel launch"); if (st) return st;
+   }
+   return hip_status(hipStreamSynchronize(0), "hipStreamSynchronize");
+}
+
 fusedMM_amd_sop_fn host_sop_function()
 {
    if (g.sop_fn) return g.sop_fn;
@@ -1260,6 +1511,57 @@ int entry(const Args &a, bool async, hipStream_t stream, int queues = kQueuesGro
    int st = make_plan(a.imessage, g.opt, &pl);
    if (st) return st;
    int sop_kind = g.sop_kind;
+   if (pl.udef_stages)
+   {
+      // stages that are the caller's host functions: registered, or found by the names the reference binds
+      StageFns f;
+      f.vop = g.vop_fn ? g.vop_fn : (fusedMM_amd_vop_fn)dlsym(RTLD_DEFAULT, "VOP_UDEF_FUNC");
+      f.rop = g.rop_fn ? g.rop_fn : (fusedMM_amd_rop_fn)dlsym(RTLD_DEFAULT, "ROP_UDEF_FUNC");
+      f.vsc = g.vsc_fn ? g.vsc_fn : (fusedMM_amd_vsc_fn)dlsym(RTLD_DEFAULT, "VSC_UDEF_FUNC");
+      f.aop = g.aop_fn ? g.aop_fn : (fusedMM_amd_aop_fn)dlsym(RTLD_DEFAULT, "AOP_UDEF_FUNC");
+      f.sop = nullptr;
+      if (((pl.udef_stages & kUdefVop) && !f.vop) || ((pl.udef_stages & kUdefRop) && !f.rop) ||
+          ((pl.udef_stages & kUdefVsc) && !f.vsc) || ((pl.udef_stages & kUdefAop) && !f.aop))
+      {
+         // what the reference's default build does with such a tuple: its stubs return this code (fusedMM_internal.h:50-84)
+         FMM_LOG("the op tuple 0x%x names a *_UDEF stage for which the process defines no <STAGE>_UDEF_FUNC "
+                 "(and none was registered with fusedMM_amd_set_stage_callbacks)", a.imessage);
+         return FUSEDMM_UNDEFINED_USER_FUNCTION;
+      }
+      if (pl.needs_sop && sop_kind == FUSEDMM_SOP_KIND_HOST && GET_VSC_FLAG(a.imessage) != VSC_NOOP)
+      {
+         f.sop = host_sop_function();
+         if (!f.sop)
+         {
+            FMM_LOG("SOP_UDEF: no host SOP_UDEF_FUNC found and no device body selected "
+                    "(fusedMM_amd_set_sop_kind / FUSEDMM_SOP_KIND)");
+            return FUSEDMM_UNDEFINED_USER_FUNCTION;
+         }
+      }
+      if (async)
+      {
+         FMM_LOG("a stage evaluated by a host function needs the synchronous entry point");
+         return FUSEDMM_UNDEFINED_USER_FUNCTION;
+      }
+      if (a.m <= 0 || a.k < 1) return FUSEDMM_SUCCESS_RETURN;
+      if (!a.val) pl.reads_val = false;
+      const int where = operand_residence(a);
+      if (where < 0) return FUSEDMM_FAIL_RETURN;
+      if (where == 1)
+      {
+         std::vector<idx_t> hb((size_t)a.m), he((size_t)a.m);
+         FMM_HIP(hipMemcpy(hb.data(), a.pntrb, (size_t)a.m * sizeof(idx_t), hipMemcpyDeviceToHost));
+         FMM_HIP(hipMemcpy(he.data(), a.pntre, (size_t)a.m * sizeof(idx_t), hipMemcpyDeviceToHost));
+         return run_host_stages(a, hb.data(), he.data(), max_slot(he.data(), a.m), pl, f, sop_kind);
+      }
+      Args dv;
+      int64_t slots = 0;
+      st = stage_up(a, pl, &dv, &slots);
+      if (st) return st;
+      st = run_host_stages(dv, a.pntrb, a.pntre, slots, pl, f, sop_kind);
+      if (st) return st;
+      return stage_down(a, dv);
+   }
    if (pl.needs_sop && sop_kind == FUSEDMM_SOP_KIND_HOST)
    {
       if (GET_VSC_FLAG(a.imessage) == VSC_NOOP)
@@ -1439,6 +1741,16 @@ void fusedMM_amd_set_sop_callback(fusedMM_amd_sop_fn fn)
 {
    std::lock_guard<std::mutex> lock(g.mu);
    g.sop_fn = fn;
+}
+
+void fusedMM_amd_set_stage_callbacks(fusedMM_amd_vop_fn vop, fusedMM_amd_rop_fn rop, fusedMM_amd_vsc_fn vsc,
+                                     fusedMM_amd_aop_fn aop)
+{
+   std::lock_guard<std::mutex> lock(g.mu);
+   g.vop_fn = vop;
+   g.rop_fn = rop;
+   g.vsc_fn = vsc;
+   g.aop_fn = aop;
 }
 
 int fusedMM_amd_set_opt(int enable)
@@ -1660,6 +1972,7 @@ void fusedMM_amd_finalize(void)
       Buffer *bufs[] = {&d.heavy, &d.segs, &d.partial, &d.queued};
       for (Buffer *b : bufs) { if (b->ptr) (void)hipFree(b->ptr); *b = Buffer(); }
       for (Buffer &b : d.stage) { if (b.ptr) (void)hipFree(b.ptr); b = Buffer(); }
+      if (d.edge_t.ptr) (void)hipFree(d.edge_t.ptr);
       for (auto &mi : d.mirrors) (void)hipFree(mi.dev);
       d.mirrors.clear();
       if (d.pin[0])

@@ -45,6 +45,33 @@ typedef int (*fusedMM_amd_sop_fn)(VALUETYPE val, VALUETYPE *out);
 void fusedMM_amd_set_sop_callback(fusedMM_amd_sop_fn fn);
 
 /*
+ * VOP_UDEF, ROP_UDEF, VSC_UDEF, AOP_UDEF: the caller's host functions, with the
+ * reference's prototypes (fusedMM.h:135-143), called as the reference calls them
+ * (fusedMM.c:696-740): VOP(k, X[i], k, Y[c], k, T); ROP(k, X[i], k, T, &scal) with
+ * scal starting as the edge value; VSC(k, T, out, k, T); AOP(k, T, k, Z[i]), the
+ * last in edge order within a row.  A tuple that names such a stage is served by
+ * the synchronous entry point when the process defines <STAGE>_UDEF_FUNC (looked up
+ * by name, as SOP_UDEF_FUNC is) or a function was registered here (NULL: look the
+ * name up); otherwise it returns FUSEDMM_UNDEFINED_USER_FUNCTION, which is what the
+ * reference's default build, compiled without <STAGE>_UDEF_IMPL, makes of it
+ * (fusedMM.h:129-133, fusedMM_internal.h:50-84).  The library's own stages of such
+ * a tuple run on the GPU, over per-edge buffers (k values per edge slot of device
+ * memory); only the caller's functions run on the host, rows dealt to a few
+ * threads, so they must be thread-safe as the reference requires
+ * (fusedMM.h:125-126).  Their return values are ignored, as in the reference's
+ * release build.
+ */
+typedef int (*fusedMM_amd_vop_fn)(INDEXTYPE lhs_dim, const VALUETYPE *lhs, INDEXTYPE rhs_dim, const VALUETYPE *rhs,
+                                  INDEXTYPE out_dim, VALUETYPE *out);
+typedef int (*fusedMM_amd_rop_fn)(INDEXTYPE lhs_dim, const VALUETYPE *lhs, INDEXTYPE rhs_dim, const VALUETYPE *rhs,
+                                  VALUETYPE *out);
+typedef int (*fusedMM_amd_vsc_fn)(INDEXTYPE rhs_dim, const VALUETYPE *rhs, VALUETYPE scal, INDEXTYPE out_dim,
+                                  VALUETYPE *out);
+typedef int (*fusedMM_amd_aop_fn)(INDEXTYPE rhs_dim, const VALUETYPE *rhs, INDEXTYPE out_dim, VALUETYPE *out);
+void fusedMM_amd_set_stage_callbacks(fusedMM_amd_vop_fn vop, fusedMM_amd_rop_fn rop, fusedMM_amd_vsc_fn vsc,
+                                     fusedMM_amd_aop_fn aop);
+
+/*
  * fusedMM_csr on a caller-supplied HIP stream: every pointer is device memory,
  * work is enqueued on `stream` (a hipStream_t; NULL is the default stream) and
  * the call returns without waiting.  No counterpart in the reference; it is what

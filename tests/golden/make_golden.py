@@ -19,6 +19,12 @@ full so nothing has to be regenerated bit-for-bit) and the reference's outputs:
                       evaluated each row on, for the degree sets of
                       graphs.partition_cases() (-1: a row without edges, whose
                       holder the reference never shows)
+  udef_stages.npz     Z of the reference's fusedMM_csr built with VOP/ROP/VSC/
+                      AOP_UDEF_IMPL switched on and linked with the caller-side
+                      stage functions of oracle/udef_stage_bodies.inc, for op
+                      tuples in which one or more stages are those functions
+                      (float and, keys ending in _d, double; int32 and int64
+                      builds agree and one copy is kept)
 """
 import os
 import sys
@@ -31,7 +37,7 @@ sys.path.insert(0, os.path.dirname(HERE))
 sys.path.insert(0, os.path.dirname(os.path.dirname(HERE)))
 
 import graphs  # noqa: E402
-from oracle_api import MSG, PARTITION_THREADS, Ref, RefPartition  # noqa: E402
+from oracle_api import MSG, PARTITION_THREADS, Ref, RefPartition, RefUdef  # noqa: E402
 
 KINDS = {"s": "sigmoid", "t": "tdist", "f": "fr", "m": "spmm", "g": "gcn"}
 
@@ -160,6 +166,28 @@ def main():
             out["%s_owner_t%d" % (name, t)] = own32.astype(np.int8)
     out["names"] = np.array(names)
     np.savez_compressed(os.path.join(HERE, "partition.npz"), **out)
+
+    # tuples with user stages through the reference built with those stages switched on
+    g = graphs.with_values(graphs.ragged(32, rows=37, cols=53, hub_deg=90))
+    k = 12
+    X = graphs.features(g["rows"], k, 9, -1, 1, 1)
+    Y = graphs.features(g["cols"], k, 9, -1, 1, 2)
+    Z0 = graphs.features(g["rows"], k, 9, -1, 1, 3)
+    out = {"pntrb": g["pntrb"], "pntre": g["pntre"], "indx": g["indx"], "val": g["val"],
+           "shape": np.array([g["rows"], g["cols"]]), "X": X, "Y": Y, "Z0": Z0}
+    msgs = graphs.udef_stage_tuples()
+    for sfx, vbits, npv in (("", 32, np.float32), ("_d", 64, np.float64)):
+        Zs = np.zeros((len(msgs),) + Z0.shape, npv)
+        g64 = dict(g, indx=g["indx"].astype(np.int64), pntrb=g["pntrb"].astype(np.int64), pntre=g["pntre"].astype(np.int64))
+        for n, imsg in enumerate(msgs):
+            Z, Zw = Z0.astype(npv), Z0.astype(npv)
+            assert RefUdef(32, vbits).fusedMM_csr(int(imsg), g, X.astype(npv), Y.astype(npv), Z) == 0
+            assert RefUdef(64, vbits).fusedMM_csr(int(imsg), g64, X.astype(npv), Y.astype(npv), Zw) == 0
+            assert np.array_equal(Z.view(np.uint8), Zw.view(np.uint8))
+            Zs[n] = Z
+        out["Z" + sfx] = Zs
+    out["msgs"] = msgs
+    np.savez_compressed(os.path.join(HERE, "udef_stages.npz"), **out)
     print("golden fixtures written to", HERE)
 
 

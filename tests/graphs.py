@@ -123,3 +123,30 @@ def partition_cases():
         pos = int(pe[r])
     cases.append(("gapped_pointers", pb, pe, 200))
     return cases
+
+
+def udef_stage_tuples():
+    """Op tuples in which at least one of VOP, ROP, VSC, AOP is a user function: every
+    single such stage with built-in neighbours of each kind, pairs, and all of them
+    together, with SOP as a copy, as a user function and absent.  (SOP_NOOP is only
+    paired with VSC_NOOP: the reference leaves the scalar uninitialised otherwise,
+    fusedMM.c:212-216.)"""
+    msgs = []
+    builtin = [(0x2, 0x10, 0x100, 0x1000, 0x10000),    # spmm-like with a dot
+               (0x5, 0x50, 0xF00, 0x1000, 0x10000),    # the distance tuple
+               (0x3, 0x00, 0x100, 0x2000, 0x20000),    # edge value as the scalar, max
+               (0x1, 0x30, 0x000, 0x0000, 0x30000),    # no scaling, min
+               (0x7, 0x20, 0xF00, 0x2000, 0x10000)]
+    udef = (0xF, 0xF0, None, 0xF000, 0xF0000)
+    for base in builtin:
+        for mask in range(1, 16):
+            stages = list(base)
+            pos = [0, 1, 3, 4]
+            for b in range(4):
+                if (mask >> b) & 1:
+                    stages[pos[b]] = udef[pos[b]]
+            if stages[2] == 0x000 and stages[3] != 0x0000:
+                continue
+            msgs.append(stages[0] | stages[1] | stages[2] | stages[3] | stages[4])
+    msgs.append(0xF | 0xF0 | 0xF00 | 0xF000 | 0x00000)   # no accumulate stage: Z untouched
+    return np.array(sorted(set(msgs)), np.int32)

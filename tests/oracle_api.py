@@ -140,6 +140,31 @@ class Oracle:
                                                   x, ldx, y, ldy, beta, z, ldz, self.cv) + [C.c_int(sop_kind)]
         return fn(*args)
 
+    def stage_fn(self, stage, bits):
+        """Address of the tests' caller-side stage function (VOP, ROP, SOP, VSC, AOP) for this
+        precision and index width (oracle/udef_stage_bodies.inc)."""
+        return C.cast(getattr(self.lib, "orc_test_%s%s_i%d" % (stage, self.sfx, bits)), C.c_void_p)
+
+    def generic_udef(self, imsg, g, x, y, z, sop_kind=0, host_sop=False, m=None, k=None, ldx=None, ldy=None, ldz=None):
+        """orc_fusedmm_generic_udef with the tests' stage functions bound to every *_UDEF
+        nibble (host_sop: also to SOP_UDEF, instead of the numbered body sop_kind)."""
+        bits = g["indx"].dtype.itemsize * 8
+        _, ct = _itype(bits)
+        m = g["rows"] if m is None else m
+        k = y.shape[1] if k is None else k
+        ldx = (x.shape[1] if x is not None else k) if ldx is None else ldx
+        ldy = y.shape[1] if ldy is None else ldy
+        ldz = z.shape[1] if ldz is None else ldz
+        fn = getattr(self.lib, "orc_fusedmm_generic_udef%s_i%d" % (self.sfx, bits))
+        fn.restype = C.c_int
+        args = [C.c_int32(imsg)] + self._csr_args(ct, m, g["cols"], k, g["nnz"], g["rows"], g["cols"],
+                                                  self._val(g), g["indx"], g["pntrb"], g["pntre"],
+                                                  x, ldx, y, ldy, 0.0, z, ldz, self.cv) + [C.c_int(sop_kind)]
+        args += [self.stage_fn("VOP", bits), self.stage_fn("ROP", bits),
+                 self.stage_fn("SOP", bits) if host_sop else C.c_void_p(None),
+                 self.stage_fn("VSC", bits), self.stage_fn("AOP", bits)]
+        return fn(*args)
+
     def opt(self, tkern, g, x, y, z, beta=0.0, sop_kind=0, mode=0, V=4, L=32, S=1, m=None, k=None,
             ldx=None, ldy=None, ldz=None, edge_s=None):
         bits = g["indx"].dtype.itemsize * 8
@@ -232,6 +257,30 @@ class Ref:
         values = np.empty(n.value, self.np_v)
         self.lib.ref_get_csr(_ptr(rowptr, self.ct), _ptr(colids, self.ct), _ptr(values, self.cv))
         return r.value, c.value, rowptr, colids, values
+
+
+def ref_udef_available(bits=32, vbits=32):
+    return os.path.exists(os.path.join(ORACLE_DIR, "_ref", _ref_name("udefstages", bits, vbits)))
+
+
+class RefUdef:
+    """The real reference's general fusedMM_csr built with VOP/ROP/VSC/AOP_UDEF_IMPL switched
+    on and linked with the tests' caller-side stage functions (oracle/ref_udef_stages.c)."""
+
+    def __init__(self, bits=32, vbits=32):
+        self.np_i, self.ct = _itype(bits)
+        self.np_v, self.cv = _vtype(vbits)
+        self.lib = C.CDLL(os.path.join(ORACLE_DIR, "_ref", _ref_name("udefstages", bits, vbits)))
+        assert self.lib.ref_udef_index_bytes() * 8 == bits and self.lib.ref_udef_value_bytes() * 8 == vbits
+
+    def fusedMM_csr(self, imsg, g, x, y, z, m=None):
+        m = g["rows"] if m is None else m
+        k = y.shape[1]
+        val = g["val"] if g["val"] is None or g["val"].dtype == self.np_v else g["val"].astype(self.np_v)
+        self.lib.fusedMM_csr.restype = C.c_int
+        args = [C.c_int32(imsg)] + Oracle._csr_args(self.ct, m, g["cols"], k, g["nnz"], g["rows"], g["cols"], val, g["indx"],
+                                                    g["pntrb"], g["pntre"], x, x.shape[1], y, k, 0.0, z, k, self.cv)
+        return self.lib.fusedMM_csr(*args)
 
 
 PARTITION_THREADS = (2, 3, 5, 8, 16)   # PART_THREADS of oracle/Makefile

@@ -189,3 +189,41 @@ def test_partition_vectors_tell_the_rule_from_its_near_misses():
             for v, kw in variants.items():
                 wrong[v] += int(not np.array_equal(_rule(deg, t, **kw)[seen], want[seen]))
     assert all(n > 0 for n in wrong.values()), wrong
+
+
+def _udef_case(d, bits, npv):
+    it = np.int32 if bits == 32 else np.int64
+    rows, cols = (int(v) for v in d["shape"])
+    g = {"rows": rows, "cols": cols, "nnz": int(d["indx"].size), "pntrb": d["pntrb"].astype(it),
+         "pntre": d["pntre"].astype(it), "indx": d["indx"].astype(it), "val": d["val"]}
+    return g, d["X"].astype(npv), d["Y"].astype(npv), d["Z0"].astype(npv)
+
+
+@pytest.mark.parametrize("bits", [32, 64])
+@pytest.mark.parametrize("vbits", [32, 64])
+def test_user_stage_tuples_bit_equal(oracle, oracle_d, bits, vbits):
+    """Tuples in which VOP, ROP, VSC or AOP (and SOP) are the caller's functions: the oracle's
+    restatement with those functions bound equals, bit for bit, what the real reference built
+    with <STAGE>_UDEF_IMPL switched on wrote for the same inputs."""
+    d = np.load(os.path.join(GOLD, "udef_stages.npz"))
+    o, npv, key = (oracle, np.float32, "Z") if vbits == 32 else (oracle_d, np.float64, "Z_d")
+    g, X, Y, Z0 = _udef_case(d, bits, npv)
+    assert len(d["msgs"]) >= 60
+    for imsg, want in zip(d["msgs"], d[key]):
+        Z = Z0.copy()
+        assert o.generic_udef(int(imsg), g, X, Y, Z, host_sop=True) == 0, hex(int(imsg))
+        np.testing.assert_array_equal(Z.view(np.uint8), want.view(np.uint8), err_msg=hex(int(imsg)))
+    # the accumulate stage is what writes Z: without one the call leaves it alone
+    i = list(d["msgs"]).index(0xFFFFF & (0xF | 0xF0 | 0xF00 | 0xF000))
+    np.testing.assert_array_equal(d[key][i], Z0)
+
+
+def test_user_stage_without_a_function_is_undefined(oracle):
+    """The reference's default build binds stubs that return FUSEDMM_UNDEFINED_USER_FUNCTION
+    (fusedMM_internal.h:50-84); the oracle reports that code and leaves Z alone."""
+    d = np.load(os.path.join(GOLD, "udef_stages.npz"))
+    g, X, Y, Z0 = _udef_case(d, 32, np.float32)
+    for imsg in (0x1110F, 0x111F2, 0x1F112, 0xF1112):
+        Z = Z0.copy()
+        assert oracle.generic(imsg, g, X, Y, Z) == 64
+        np.testing.assert_array_equal(Z, Z0)

@@ -97,3 +97,35 @@ def test_partition_rows_live(oracle, bits, nthreads):
         got = owners_from_ranges(rb, re, m)
         seen = want >= 0
         assert got.min() >= 0 and np.array_equal(got[seen], want[seen]), (rep, n, m)
+
+
+@pytest.mark.parametrize("bits,vbits", [(32, 32), (64, 32), (32, 64), (64, 64)])
+def test_user_stage_tuples_live(bits, vbits):
+    """Every tuple with a user stage (1344 of them: all built-in neighbours, every precision
+    and index width) through the real reference built with <STAGE>_UDEF_IMPL switched on and
+    through the oracle's restatement bound to the same caller-side functions: same status,
+    same bits.  (SOP_NOOP with a scaling stage is left out: the reference passes an
+    uninitialised scalar there, fusedMM.c:212-216.)"""
+    import itertools
+    from oracle_api import Oracle, RefUdef, ref_udef_available
+    if not ref_udef_available(bits, vbits):
+        pytest.skip("oracle/_ref/libref_udefstages not built")
+    npv = np.float32 if vbits == 32 else np.float64
+    o, r = Oracle(vbits=vbits), RefUdef(bits, vbits)
+    g = graphs.with_values(graphs.ragged(bits, seed=17, hub_deg=70))
+    k = 20
+    X = graphs.features(g["rows"], k, 5, -0.5, 0.5, 1).astype(npv)
+    Y = graphs.features(g["cols"], k, 5, -0.5, 0.5, 2).astype(npv)
+    Z0 = graphs.features(g["rows"], k, 5, -1, 1, 3).astype(npv)
+    n = 0
+    for v, rp, sp, vs, ap in itertools.product((1, 2, 3, 4, 5, 6, 7, 0xF), (0x00, 0x10, 0x20, 0x30, 0x40, 0x50, 0xF0),
+                                               (0x000, 0x100, 0xF00), (0x0000, 0x1000, 0x2000, 0xF000),
+                                               (0x00000, 0x10000, 0x20000, 0x30000, 0xF0000)):
+        if not (v == 0xF or rp == 0xF0 or vs == 0xF000 or ap == 0xF0000) or (sp == 0x000 and vs != 0x0000):
+            continue
+        msg = v | rp | sp | vs | ap
+        za, zb = Z0.copy(), Z0.copy()
+        assert r.fusedMM_csr(msg, g, X, Y, za) == o.generic_udef(msg, g, X, Y, zb, host_sop=True) == 0, hex(msg)
+        assert np.array_equal(za.view(np.uint8), zb.view(np.uint8)), hex(msg)
+        n += 1
+    assert n == 1344
