@@ -20,6 +20,15 @@
  *   orc_fusedmm_generic_*  - bit-compared with the reference's generic
  *          fusedMM_csr (compiled from /root/reference/fusedMM.c) on seeded
  *          inputs; scipy CSR @ Y for the spmm/gcn tuples; dense brute force.
+ *   orc_fusedmm_generic_udef_* (the general pipeline with the caller's VOP / ROP /
+ *          SOP / VSC / AOP functions bound) - bit-compared with the reference's
+ *          fusedMM.c built with VOP/ROP/VSC/AOP_UDEF_IMPL switched on and linked with
+ *          the same caller-side functions (ref_udef_stages.c, udef_stage_bodies.inc):
+ *          all 1344 tuples with a user stage, live, in every precision and index
+ *          width (tests/test_oracle_ref.py), 65 of them committed as
+ *          tests/golden/udef_stages.npz.  The functions are asymmetric, use the
+ *          scalar's start value, work in place and do not commute across edges, so
+ *          swapped operands, a missing seed or a changed edge order show.
  *   orc_fusedmm_opt_*      - golden Z from the reference harness's trusted
  *          kernels and generic fusedMM_csr; dense fp64 brute force; invariants.
  *   orc_partition_rows_*   - row for row against the thread the real reference
