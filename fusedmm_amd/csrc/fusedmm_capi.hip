@@ -1319,11 +1319,6 @@ int run_host_stages(const Args &a, const idx_t *h_pb, const idx_t *h_pe, int64_t
    if (slots <= 0) return FUSEDMM_SUCCESS_RETURN;   // no processed row has an edge: Z is left alone (general rule)
    const int vop = GET_VOP_FLAG(a.imessage), rop = GET_ROP_FLAG(a.imessage), sop = GET_SOP_FLAG(a.imessage),
              vsc = GET_VSC_FLAG(a.imessage), aop = GET_AOP_FLAG(a.imessage);
-   if ((pl.udef_stages & kUdefVop) && a.n <= 0)
-   {
-      FMM_LOG("VOP_UDEF: n must be the number of rows of Y (the host function is handed rows of a host copy of Y)");
-      return FUSEDMM_FAIL_RETURN;
-   }
    const int64_t m = a.m, k = a.k;
    const size_t nT = (size_t)slots * (size_t)k;
    st = grow(d->edge_t, nT * kValBytes); if (st) return st;
@@ -1381,10 +1376,27 @@ int run_host_stages(const Args &a, const idx_t *h_pb, const idx_t *h_pe, int64_t
    if (pl.udef_stages & kUdefVop)
    {
       st = need_X_host(); if (st) return st;
-      hY.resize((size_t)(a.n - 1) * (size_t)a.ldy + (size_t)k);
-      FMM_HIP(hipMemcpy(hY.data(), a.y, hY.size() * kValBytes, hipMemcpyDeviceToHost));
       hidx.resize((size_t)slots);
       FMM_HIP(hipMemcpy(hidx.data(), a.indx, (size_t)slots * sizeof(idx_t), hipMemcpyDeviceToHost));
+      // the host function is handed rows of a host copy of Y: as many rows as the processed edges reach
+      // (n is not trusted: the reference never reads it)
+      int64_t y_rows = 0;
+      for (int64_t i = 0; i < m; i++)
+         for (int64_t j = (int64_t)h_pb[i]; j < (int64_t)h_pe[i]; j++)
+         {
+            const int64_t c = (int64_t)hidx[(size_t)j];
+            if (c < 0)
+            {
+               FMM_LOG("negative column id %lld in row %lld", (long long)c, (long long)i);
+               return FUSEDMM_FAIL_RETURN;
+            }
+            if (c >= y_rows) y_rows = c + 1;
+         }
+      if (y_rows > 0)
+      {
+         hY.resize((size_t)(y_rows - 1) * (size_t)a.ldy + (size_t)k);
+         FMM_HIP(hipMemcpy(hY.data(), a.y, hY.size() * kValBytes, hipMemcpyDeviceToHost));
+      }
       hT.assign(nT, (val_t)0);
       for_row_ranges(m, [&](int64_t lo, int64_t hi) {
          for (int64_t i = lo; i < hi; i++)
