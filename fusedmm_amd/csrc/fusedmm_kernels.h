@@ -904,25 +904,77 @@ __device__ __forceinline__ int64_t resolve_claim(const Params<IdxT> &p, unsigned
 // heavy_deg edges gets a HeavyRow entry and one SegDesc per segment (at most
 // kMaxSegsPerRow: hub rows get longer segments) and its bit in `queued` is set.
 // When the queue is full the row is left for phase B to process whole.
+//
+// Queue entries are handed out by a 64-bit read-modify-write on n_heavy (low word)
+// and n_seg (high word), which advance together.  Read-modify-writes on that one
+// cache line retire one per ~12 ns however many CUs issue them (13 000 heavy rows of
+// an R-MAT graph taking it one by one: 0.2 ms; one per wavefront and 64 rows: 0.15 ms),
+// so a workgroup first collects the heavy rows among all the rows it looks at in LDS
+// and then takes the counters once for all of them.
+constexpr int kClassifyList = 512;   // heavy rows a workgroup collects; more are queued one by one
+
+template <typename IdxT>
+__device__ __forceinline__ unsigned int segments_of(const Params<IdxT> &p, int64_t deg, int64_t *seg_len_out)
+{
+   int64_t seg_len = p.seg_len;
+   if (deg > seg_len * (int64_t)kMaxSegsPerRow) seg_len = (deg + kMaxSegsPerRow - 1) / kMaxSegsPerRow;
+   *seg_len_out = seg_len;
+   return (unsigned int)((deg + seg_len - 1) / seg_len);
+}
+
+// Entry `slot` of the heavy-row queue and its segment descriptors [base, base + nseg), written by the
+// threads tid, tid + nthreads, ... of the caller's group; or, when the queue is full, the entry
+// poisoned (the merge kernel skips n_seg == 0; every queue entry below the cap has exactly one writer).
+template <typename IdxT>
+__device__ __forceinline__ void write_queue_entry(const Params<IdxT> &p, unsigned int slot, unsigned int base, unsigned int nseg,
+                                                  int64_t row, int64_t jb, int64_t deg, int64_t seg_len, int tid, int nthreads)
+{
+   if (slot < p.cap_heavy && (uint64_t)base + nseg <= (uint64_t)p.cap_seg)
+   {
+      if (tid == 0)
+      {
+         p.heavy[slot] = HeavyRow{row, base, nseg};
+         atomicOr(&p.queued[row >> 5], 1u << (row & 31));
+      }
+      for (unsigned int s = (unsigned int)tid; s < nseg; s += (unsigned int)nthreads)
+      {
+         const int64_t off = (int64_t)s * seg_len;
+         const int64_t cnt = deg - off < seg_len ? deg - off : seg_len;
+         p.segs[base + s] = SegDesc{row, jb + off, (unsigned int)cnt, 0u};
+      }
+   }
+   else
+   {
+      if (tid == 0)
+      {
+         if (slot < p.cap_heavy) p.heavy[slot] = HeavyRow{row, 0u, 0u};
+         atomicAdd(&p.ctr->overflow, 1u);
+      }
+      for (uint64_t s = (uint64_t)base + (unsigned int)tid; s < (uint64_t)base + nseg && s < (uint64_t)p.cap_seg; s += (unsigned int)nthreads)
+         p.segs[s] = SegDesc{-1, 0, 0u, 0u};
+   }
+}
+
 template <typename IdxT>
 __global__ __launch_bounds__(kBlockThreads) void classify_kernel(const Params<IdxT> p)
 {
-   const int lane = threadIdx.x & 63;
+   __shared__ int64_t l_row[kClassifyList], l_jb[kClassifyList], l_deg[kClassifyList];
+   __shared__ unsigned int l_base[kClassifyList];
+   __shared__ unsigned int l_scan[kBlockThreads];
+   __shared__ unsigned int l_count;
+   __shared__ unsigned long long l_before;
+   const int tid = threadIdx.x, lane = threadIdx.x & 63;
    const int64_t stride = (int64_t)gridDim.x * kBlockThreads;
-   // Queue entries are handed out by ONE 64-bit read-modify-write per wavefront and
-   // turn: n_heavy (low word) and n_seg (high word) advance together, by the number of
-   // heavy rows among the wave's 64 rows and by the sum of their segment counts.  Every
-   // heavy row taking the two counters by itself made this pass wait ~12 ns per
-   // read-modify-write on the one cache line (13 000 heavy rows of an R-MAT graph: 0.2 ms).
    unsigned long long *both = reinterpret_cast<unsigned long long *>(&p.ctr->n_heavy);
-   auto queue_rows = [&](int64_t row, IdxT jb, IdxT je) {
-      const int64_t deg = (int64_t)je - (int64_t)jb;
-      const bool heavy = deg > p.heavy_deg;
-      const unsigned long long mask = __ballot(heavy);
-      if (mask == 0ull) return;                                    // wave-uniform
+   if (tid == 0) l_count = 0u;
+   __syncthreads();
+
+   // A wavefront that finds many heavy rows among its 64 (R-MAT degrees follow the bits
+   // of the row id, so they come in runs) takes the counters for all of them at once;
+   // a few here and there go on the workgroup's list.  All lanes call this together.
+   auto wave_takes_counters = [&](int64_t row, int64_t jb, int64_t deg, bool heavy, unsigned long long mask) {
       int64_t seg_len = p.seg_len;
-      if (deg > seg_len * (int64_t)kMaxSegsPerRow) seg_len = (deg + kMaxSegsPerRow - 1) / kMaxSegsPerRow;
-      const unsigned int nseg = heavy ? (unsigned int)((deg + seg_len - 1) / seg_len) : 0u;
+      const unsigned int nseg = heavy ? segments_of(p, deg, &seg_len) : 0u;
       unsigned int incl = nseg;                                    // inclusive prefix sum of nseg over the lanes
 #pragma unroll
       for (int d = 1; d < 64; d <<= 1)
@@ -938,33 +990,15 @@ __global__ __launch_bounds__(kBlockThreads) void classify_kernel(const Params<Id
       before = __shfl(before, leader, 64);
       if (!heavy) return;
       const unsigned int slot = (unsigned int)(before & 0xFFFFFFFFull) + (unsigned int)__builtin_popcountll(mask & ((1ull << lane) - 1ull));
-      const unsigned int base = (unsigned int)(before >> 32) + (incl - nseg);
-      if (slot < p.cap_heavy && (uint64_t)base + nseg <= (uint64_t)p.cap_seg)
-      {
-         p.heavy[slot] = HeavyRow{row, base, nseg};
-         for (unsigned int s = 0; s < nseg; s++)
-         {
-            const int64_t off = (int64_t)s * seg_len;
-            const int64_t cnt = deg - off < seg_len ? deg - off : seg_len;
-            p.segs[base + s] = SegDesc{row, (int64_t)jb + off, (unsigned int)cnt, 0u};
-         }
-         atomicOr(&p.queued[row >> 5], 1u << (row & 31));
-      }
-      else
-      {
-         // slot unused (the merge kernel skips n_seg == 0); every queue entry below the
-         // cap has exactly one writer: poison ours
-         if (slot < p.cap_heavy) p.heavy[slot] = HeavyRow{row, 0u, 0u};
-         atomicAdd(&p.ctr->overflow, 1u);
-         for (uint64_t s = base; s < (uint64_t)base + nseg && s < (uint64_t)p.cap_seg; s++)
-            p.segs[s] = SegDesc{-1, 0, 0u, 0u};
-      }
+      write_queue_entry(p, slot, (unsigned int)(before >> 32) + (incl - nseg), nseg, row, jb, deg, seg_len, 0, 1);
    };
+   constexpr int kManyInAWave = 8;
+
    // four rows per thread and turn, their pointers requested together; the turn's
    // bounds are the wave's (its first lane's row), so that every lane takes part in
-   // the wave-wide steps above
+   // the wave-wide steps
    constexpr int kRowsPerTurn = 4;
-   for (int64_t row0 = (int64_t)blockIdx.x * kBlockThreads + threadIdx.x; row0 - lane < p.m; row0 += kRowsPerTurn * stride)
+   for (int64_t row0 = (int64_t)blockIdx.x * kBlockThreads + tid; row0 - lane < p.m; row0 += kRowsPerTurn * stride)
    {
       IdxT jb[kRowsPerTurn], je[kRowsPerTurn];
 #pragma unroll
@@ -975,7 +1009,87 @@ __global__ __launch_bounds__(kBlockThreads) void classify_kernel(const Params<Id
          je[i] = row < p.m ? p.pntre[row] : (IdxT)0;
       }
 #pragma unroll
-      for (int i = 0; i < kRowsPerTurn; i++) queue_rows(row0 + i * stride, jb[i], je[i]);
+      for (int i = 0; i < kRowsPerTurn; i++)
+      {
+         const int64_t row = row0 + i * stride;
+         const int64_t deg = (int64_t)je[i] - (int64_t)jb[i];
+         const bool heavy = deg > p.heavy_deg;
+         const unsigned long long mask = __ballot(heavy);
+         if (mask == 0ull) continue;                               // wave-uniform
+         const int found = __builtin_popcountll(mask);
+         bool listed = false;
+         if (found < kManyInAWave)
+         {
+            const int leader = __builtin_ctzll(mask);
+            unsigned int at0 = 0xFFFFFFFFu;
+            if (lane == leader)
+            {
+               unsigned int seen = l_count;
+               while (seen + (unsigned int)found <= (unsigned int)kClassifyList)
+               {
+                  const unsigned int was = atomicCAS(&l_count, seen, seen + (unsigned int)found);
+                  if (was == seen) { at0 = seen; break; }
+                  seen = was;
+               }
+            }
+            at0 = (unsigned int)__shfl((int)at0, leader, 64);
+            if (at0 != 0xFFFFFFFFu)                                // room on the list
+            {
+               if (heavy)
+               {
+                  const unsigned int at = at0 + (unsigned int)__builtin_popcountll(mask & ((1ull << lane) - 1ull));
+                  l_row[at] = row; l_jb[at] = (int64_t)jb[i]; l_deg[at] = deg;
+               }
+               listed = true;
+            }
+         }
+         if (!listed) wave_takes_counters(row, (int64_t)jb[i], deg, heavy, mask);
+      }
+   }
+   __syncthreads();
+   const unsigned int n = l_count;                                 // <= kClassifyList
+   if (n == 0u) return;                                            // uniform over the workgroup
+
+   // thread tid owns entries kPerThread * tid + i; exclusive prefix of their segment counts over the list
+   constexpr int kPerThread = kClassifyList / kBlockThreads;
+   unsigned int mine[kPerThread], sum = 0u;
+#pragma unroll
+   for (int i = 0; i < kPerThread; i++)
+   {
+      const unsigned int e = (unsigned int)(tid * kPerThread + i);
+      int64_t seg_len;
+      mine[i] = e < n ? segments_of(p, l_deg[e], &seg_len) : 0u;
+      sum += mine[i];
+   }
+   l_scan[tid] = sum;
+   __syncthreads();
+   for (int d = 1; d < kBlockThreads; d <<= 1)                     // inclusive scan of the threads' sums
+   {
+      const unsigned int add = tid >= d ? l_scan[tid - d] : 0u;
+      __syncthreads();
+      l_scan[tid] += add;
+      __syncthreads();
+   }
+   if (tid == kBlockThreads - 1) l_before = atomicAdd(both, (unsigned long long)n | ((unsigned long long)l_scan[tid] << 32));
+   __syncthreads();
+   const unsigned int slot0 = (unsigned int)(l_before & 0xFFFFFFFFull), base0 = (unsigned int)(l_before >> 32);
+   {
+      unsigned int b = base0 + l_scan[tid] - sum;                  // first segment slot of this thread's first entry
+#pragma unroll
+      for (int i = 0; i < kPerThread; i++)
+      {
+         const unsigned int e = (unsigned int)(tid * kPerThread + i);
+         if (e < n) l_base[e] = b;
+         b += mine[i];
+      }
+   }
+   __syncthreads();
+   // an entry per wavefront at a time, its segment descriptors dealt to the lanes
+   for (unsigned int e = (unsigned int)(tid >> 6); e < n; e += (unsigned int)kWavesPerBlock)
+   {
+      int64_t seg_len;
+      const unsigned int nseg = segments_of(p, l_deg[e], &seg_len);
+      write_queue_entry(p, slot0 + e, l_base[e], nseg, l_row[e], l_jb[e], l_deg[e], seg_len, lane, 64);
    }
 }
 
