@@ -201,6 +201,8 @@ def main():
                          "timed region samples rather than instruments every step")
     ap.add_argument("--read-probe", action="store_true",
                     help="also time a read-only stream over 4 GiB (what HBM delivers to reads alone) and report it")
+    ap.add_argument("--ldz", type=int, default=0,
+                    help="leading dimension of Z in elements (default K): rows of Z further apart in memory")
     ap.add_argument("--gather-probe", action="store_true",
                     help="also time a read-only gather of uniformly random rows of the workload's row size from a buffer "
                          "the size of its Y (what the memory system delivers to such gathers alone) and report it")
@@ -243,11 +245,12 @@ def main():
     d_val, d_indx, d_pb, d_pe = up(g["val"]), up(g["indx"]), up(g["pntrb"]), up(g["pntre"])
     d_X = up(X)
     d_Y = d_X if Y is X else up(Y)
-    d_Z = torch.zeros((m, k), dtype=torch.float32 if vbits == 32 else torch.float64, device=dev)
+    ldz = max(k, args.ldz)
+    d_Z = torch.zeros((m, ldz), dtype=torch.float32 if vbits == 32 else torch.float64, device=dev)
     stream = torch.cuda.current_stream().cuda_stream
 
     def step():
-        rc = fa.fusedMM_csr(imsg, m, n, k, 1.0, nnz, m, n, d_val, d_indx, d_pb, d_pe, d_X, k, d_Y, k, 0.0, d_Z, k,
+        rc = fa.fusedMM_csr(imsg, m, n, k, 1.0, nnz, m, n, d_val, d_indx, d_pb, d_pe, d_X, k, d_Y, k, 0.0, d_Z, ldz,
                             index_bits=bits, stream=stream, value_bits=vbits)
         if rc != 0:
             raise SystemExit("fusedMM_csr returned %d" % rc)
@@ -377,7 +380,7 @@ def main():
         # (the general pipeline's tolerance check holds a row's terms in double precision: rows to 10^5 edges)
         if deg[hub] <= (100000 if args.general else 1200000):
             windows.append((hub, hub + 1))
-        z_all = d_Z.cpu().numpy() if m * k <= (1 << 28) else None
+        z_all = d_Z[:, :k].cpu().numpy() if m * ldz <= (1 << 28) else None
         checked = True
         for lo, hi in windows:
             sub = dict(g)
@@ -385,7 +388,8 @@ def main():
             Xs = None if X is None else X[lo:hi]
             want = oracle_mirror(orc, tkern, sub, Xs, Y, np.zeros((hi - lo, k), np_v), 0.0, kind_id, k,
                                  heavy_deg, seg_len)
-            got = z_all[lo:hi] if z_all is not None else d_Z[lo:hi].cpu().numpy()
+            got = z_all[lo:hi] if z_all is not None else d_Z[lo:hi, :k].cpu().numpy()
+            got = np.ascontiguousarray(got)
             if not args.general:
                 checked = checked and bool(np.array_equal(got.view(np.uint8), want.view(np.uint8)))
                 continue
@@ -418,7 +422,7 @@ def main():
         "dtype": args.dtype, "data": "synthetic",
         "config": {"workload": "%s: %s" % (args.workload, desc), "op": tkern, "K": k, "rows": m, "nnz": nnz,
                    "index_bits": bits, "beta": 0.0, "graph_gen_s": round(t_gen, 2),
-                   "pipeline": "general" if args.general else "optimised"},
+                   "pipeline": "general" if args.general else "optimised", "ldz": ldz},
         "edges_per_s": nnz / (ms_per_step * 1e-3),
         "hbm_GBps_algorithmic": b_alg / (ms_per_step * 1e-3) / 1e9,
         "pct_peak_hbm": 100.0 * b_alg / (ms_per_step * 1e-3) / 1e9 / PEAK_HBM_GBPS,
