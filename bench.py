@@ -339,6 +339,9 @@ def main():
     # bytes are quoted on the three together (classify_kernel only reads row pointers).
     hs = (C.c_uint(), C.c_uint(), C.c_uint())
     lib.fusedMM_amd_last_split(C.byref(hs[0]), C.byref(hs[1]), C.byref(hs[2]))
+    ro = (C.c_int(), C.c_uint(), C.c_uint())
+    lib.fusedMM_amd_last_row_order(C.byref(ro[0]), C.byref(ro[1]), C.byref(ro[2]))
+    row_order = {"scattered": bool(ro[0].value), "sampled_edges_lower_half": ro[1].value, "sampled_edges_upper_half": ro[2].value}
     split = hs[1].value > 0
     dom_ms = kern_ms["fused_kernel"] + (kern_ms["merge_kernel"] + kern_ms["classify_kernel"] if split else 0.0)
     if ncalls <= 0:
@@ -431,6 +434,7 @@ def main():
         "kernels_ms_per_call": {"min": float(np.min(per_call)), "median": float(np.median(per_call)),
                                 "max": float(np.max(per_call))} if per_call else None,
         "split": {"heavy_rows": hs[0].value, "segments": hs[1].value, "overflow": hs[2].value},
+        "row_order": row_order,
         "spot_check_vs_oracle": checked,
         "roofline": roofline,
     }

@@ -37,7 +37,7 @@ EXPORTS = ("fusedMM_csr", "fusedMM_csr_stream", "fusedMM_csr_stream_noalloc", "f
            "fusedMM_amd_set_sop_kind", "fusedMM_amd_get_sop_kind", "fusedMM_amd_set_sop_callback",
            "fusedMM_amd_set_opt", "fusedMM_amd_set_validate", "fusedMM_amd_set_split", "fusedMM_amd_timing",
            "fusedMM_amd_timing_summary", "fusedMM_amd_timing_call", "fusedMM_amd_last_split", "fusedMM_amd_copy_probe",
-           "fusedMM_amd_read_probe", "fusedMM_amd_gather_probe", "fusedMM_amd_set_stage_callbacks", "fusedMM_amd_set_cache", "fusedMM_amd_invalidate", "fusedMM_amd_last_host_phases",
+           "fusedMM_amd_read_probe", "fusedMM_amd_gather_probe", "fusedMM_amd_last_row_order", "fusedMM_amd_set_stage_callbacks", "fusedMM_amd_set_cache", "fusedMM_amd_invalidate", "fusedMM_amd_last_host_phases",
            "fusedMM_amd_finalize")
 
 _libs = {}
@@ -99,6 +99,8 @@ def load(index_bits=32, value_bits=32):
     lib.fusedMM_amd_read_probe.restype = C.c_int
     lib.fusedMM_amd_gather_probe.argtypes = [vp, C.c_int, vp, C.c_int64, C.c_int, C.c_int, C.c_int, vp, vp]
     lib.fusedMM_amd_gather_probe.restype = C.c_int
+    lib.fusedMM_amd_last_row_order.argtypes = [vp, vp, vp]
+    lib.fusedMM_amd_last_row_order.restype = C.c_int
     lib.fusedMM_amd_set_stage_callbacks.argtypes = [vp, vp, vp, vp]
     lib.fusedMM_amd_set_stage_callbacks.restype = None
     lib.fusedMM_amd_set_cache.argtypes = [C.c_int]

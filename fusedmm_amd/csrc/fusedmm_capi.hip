@@ -1900,6 +1900,22 @@ int fusedMM_amd_last_split(unsigned int *heavy_rows, unsigned int *segments, uns
    return FUSEDMM_SUCCESS_RETURN;
 }
 
+int fusedMM_amd_last_row_order(int *scattered, unsigned int *edges_lower_half, unsigned int *edges_upper_half)
+{
+   std::lock_guard<std::mutex> lock(g.mu);
+   DeviceState *d = nullptr;
+   int st = device_basics(&d);
+   if (st) return st;
+   Counters c;
+   memset(&c, 0, sizeof(c));
+   FMM_HIP(hipDeviceSynchronize());
+   if (d->last_ctr) FMM_HIP(hipMemcpy(&c, d->last_ctr, sizeof(c), hipMemcpyDeviceToHost));
+   if (scattered) *scattered = (int)c.last_scattered;
+   if (edges_lower_half) *edges_lower_half = (unsigned int)(c.last_skew & 0xFFFFFFFFull);
+   if (edges_upper_half) *edges_upper_half = (unsigned int)(c.last_skew >> 32);
+   return FUSEDMM_SUCCESS_RETURN;
+}
+
 int fusedMM_amd_copy_probe(void *dst, const void *src, int64_t bytes, void *stream)
 {
    if (!dst || !src || bytes < 16 || (bytes & 15) || !aligned16(dst) || !aligned16(src)) return FUSEDMM_FAIL_RETURN;

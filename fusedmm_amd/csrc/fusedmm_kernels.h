@@ -64,7 +64,14 @@ struct Counters {
    unsigned int invalid;    // set by the optional operand check
    unsigned int last_heavy, last_seg, last_overflow;   // n_heavy, n_seg, overflow of the call that finished last
    unsigned int merge_heavy;      // heavy rows the merge kernel of this call has to fold (n_heavy, capped)
-   unsigned int pad2[23];         // keep the row counters on their own 128-byte lines
+   unsigned int pad1;
+   // Edges of rows that are not split, in the lower (low word) and upper half of the row space, over a sample
+   // of the rows and scaled down, left by the classify kernel: tells the fused kernel whether the row phase's
+   // work is spread evenly along the rows.
+   unsigned long long skew;
+   unsigned long long last_skew;  // skew of the call that finished last
+   unsigned int last_scattered;   // 1: that call's row phase took the stretches of the row space in scattered order
+   unsigned int pad2[17];         // keep the row counters on their own 128-byte lines
    // Row claim counters.  Read-modify-writes on ONE address retire one per
    // ~12 ns on this GPU however many CUs issue them; on distinct 128-byte
    // lines they proceed in parallel.  So the row space is dealt to
@@ -871,6 +878,18 @@ __device__ __forceinline__ lds_table_t stage_table(const real_t *gtab, real_t *l
    return (lds_table_t)lds;      // read only when `need` held
 }
 
+// Does the row phase take the stretches of 64 chunks in scattered order?  When rows are claimed dynamically,
+// there are stretches to permute, and one half of the row space holds more than 1.25 times the other's
+// edges (the classify kernel's sample; 1.0 +- a few per cent where degrees do not follow the row id).
+template <typename IdxT>
+__device__ __forceinline__ bool scattered_order(const Params<IdxT> &p)
+{
+   const int64_t nchunks = (p.m + kRowsPerClaim - 1) / kRowsPerClaim;
+   const unsigned long long skew = p.ctr->skew;
+   const unsigned long long e_lo = skew & 0xFFFFFFFFull, e_hi = skew >> 32;
+   return p.row_counters > 0 && (nchunks >> 6) > 1 && (4 * e_lo > 5 * e_hi || 4 * e_hi > 5 * e_lo);
+}
+
 // Turn the value an atomicAdd on counter `cur` returned (in lane 0) into a
 // chunk id, moving to another counter when this one is used up.  Returns -1
 // when every counter is used up; counters only grow, so every wave gets there.
@@ -966,8 +985,13 @@ __global__ __launch_bounds__(kBlockThreads) void classify_kernel(const Params<Id
    const int tid = threadIdx.x, lane = threadIdx.x & 63;
    const int64_t stride = (int64_t)gridDim.x * kBlockThreads;
    unsigned long long *both = reinterpret_cast<unsigned long long *>(&p.ctr->n_heavy);
-   if (tid == 0) l_count = 0u;
+   __shared__ unsigned long long l_edges[2];   // edges of this workgroup's rows in the lower / upper half of the row space
+   if (tid == 0) { l_count = 0u; l_edges[0] = 0ull; l_edges[1] = 0ull; }
    __syncthreads();
+   // 32 workgroups spread evenly over the grid (all of a small grid) report where the edges of their rows lie
+   const unsigned int sample_step = gridDim.x >= 64u ? gridDim.x / 32u : 1u;
+   const bool sampled = blockIdx.x % sample_step == 0u;
+   unsigned long long edges_lo = 0ull, edges_hi = 0ull;
 
    // A wavefront that finds many heavy rows among its 64 (R-MAT degrees follow the bits
    // of the row id, so they come in runs) takes the counters for all of them at once;
@@ -1013,6 +1037,12 @@ __global__ __launch_bounds__(kBlockThreads) void classify_kernel(const Params<Id
       {
          const int64_t row = row0 + i * stride;
          const int64_t deg = (int64_t)je[i] - (int64_t)jb[i];
+         if (sampled && deg > 0 && deg <= p.heavy_deg)              // rows the row phase will walk
+         {
+            const bool upper = 2 * row >= p.m;
+            edges_lo += upper ? 0ull : (unsigned long long)deg;
+            edges_hi += upper ? (unsigned long long)deg : 0ull;
+         }
          const bool heavy = deg > p.heavy_deg;
          const unsigned long long mask = __ballot(heavy);
          if (mask == 0ull) continue;                               // wave-uniform
@@ -1046,7 +1076,24 @@ __global__ __launch_bounds__(kBlockThreads) void classify_kernel(const Params<Id
          if (!listed) wave_takes_counters(row, (int64_t)jb[i], deg, heavy, mask);
       }
    }
+   if (sampled)
+   {
+#pragma unroll
+      for (int d = 32; d >= 1; d >>= 1)                            // wave sums, then one LDS update per wave
+      {
+         edges_lo += (unsigned long long)__shfl_xor((long long)edges_lo, d, 64);
+         edges_hi += (unsigned long long)__shfl_xor((long long)edges_hi, d, 64);
+      }
+      if (lane == 0 && edges_lo) atomicAdd(&l_edges[0], edges_lo);
+      if (lane == 0 && edges_hi) atomicAdd(&l_edges[1], edges_hi);
+   }
    __syncthreads();
+   if (sampled && tid == 0)
+   {
+      // both halves in one word, scaled down so that neither can wrap
+      const unsigned long long lo = l_edges[0] >> 6, hi = l_edges[1] >> 6;
+      if (lo | hi) atomicAdd(&p.ctr->skew, (lo & 0xFFFFFFFFull) | (hi << 32));
+   }
    const unsigned int n = l_count;                                 // <= kClassifyList
    if (n == 0u) return;                                            // uniform over the workgroup
 
@@ -1161,6 +1208,7 @@ __device__ __forceinline__ void segments_phase(const Params<IdxT> &p, lds_table_
    }
 }
 
+
 // ---- phase B of the fused kernel: one wavefront per row ---------------------------
 template <int V, int L, int R, bool EXACT, int OP, int SOPK, int U, typename IdxT>
 __device__ __forceinline__ void rows_phase(const Params<IdxT> &p, lds_table_t tab)
@@ -1183,6 +1231,9 @@ __device__ __forceinline__ void rows_phase(const Params<IdxT> &p, lds_table_t ta
    // wave w simply takes chunk w -- nothing to balance, no counter traffic.
    const int nc = p.row_counters;                        // 64, 1 for tiny grids, 0: static
    const int64_t nchunks = (p.m + kRowsPerClaim - 1) / kRowsPerClaim;
+   // one half of the row space holds more than 1.5 times the edges of the other (classify kernel's sample)
+   const int64_t stretches = nchunks >> 6;
+   const bool scatter = scattered_order(p);
    const int64_t wave_id = (int64_t)blockIdx.x * kWavesPerBlock + (threadIdx.x >> 6);
    int cur = nc > 0 ? (int)(wave_id & (unsigned)(nc - 1)) : 0;
    unsigned long long claimed = 0;
@@ -1195,7 +1246,14 @@ __device__ __forceinline__ void rows_phase(const Params<IdxT> &p, lds_table_t ta
    }
    while (chunk >= 0)
    {
-   const int64_t row0 = chunk * kRowsPerClaim;
+   // Where the rows' work follows their position (R-MAT degrees follow the bits of the row id; vertices
+   // sorted by degree), stretches of 64 chunks are taken in a scattered order, so that what the GPU works
+   // on at any time is a mix of the whole row space rather than one stretch of it, all dense or all
+   // nearly empty.  The map is one-to-one: the multiplier is a prime larger than any number of stretches.
+   int64_t at = chunk;
+   if (scatter && (chunk >> 6) < stretches)
+      at = (int64_t)(((unsigned long long)(chunk >> 6) * 2654435761ull) % (unsigned long long)stretches) * 64 + (chunk & 63);
+   const int64_t row0 = at * kRowsPerClaim;
    IdxT my_b = 0, my_e = 0;   // lane t holds the pointers of row0 + t
    if (lane < kRowsPerClaim && row0 + lane < p.m)
    {
@@ -1347,6 +1405,9 @@ __device__ __forceinline__ void retire_wave(const Params<IdxT> &p)
       c->n_seg = 0u;
       c->overflow = 0u;
       c->done_groups = 0u;
+      c->last_skew = c->skew;
+      c->last_scattered = scattered_order(p) ? 1u : 0u;
+      c->skew = 0ull;
    }
 }
 

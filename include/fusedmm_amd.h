@@ -226,6 +226,15 @@ int fusedMM_amd_timing_call(int i, double *classify_ms, double *fused_ms, double
  * segments queued, heavy rows that did not fit the queue.  Waits for the device. */
 int fusedMM_amd_last_split(unsigned int *heavy_rows, unsigned int *segments, unsigned int *overflow);
 
+/* Where the last call's rows (those not split into segments) had their edges, as its first kernel
+ * sampled it (the rows of 32 of its workgroups, scaled down by 64): in the lower and in the upper half
+ * of the row space.  When one half holds
+ * more than 1.25 times the other (R-MAT graphs, vertices sorted by degree) and rows are claimed
+ * dynamically, `scattered` is 1: the row phase then took stretches of 512 rows in a scattered order
+ * instead of first to last, so that the GPU works on a mix of dense and sparse rows at any time.
+ * Results do not depend on it.  Waits for the GPU. */
+int fusedMM_amd_last_row_order(int *scattered, unsigned int *edges_lower_half, unsigned int *edges_upper_half);
+
 /* Copy `bytes` (a multiple of 16, device memory, 16-byte aligned) with a plain
  * grid-stride kernel on `stream`, asynchronously.  A measuring aid: hardware
  * traffic counters of the kernels are scaled by what they read for this copy

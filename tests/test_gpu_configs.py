@@ -35,6 +35,39 @@ def test_scaled_config_equals_oracle(oracle, name, sd):
         assert np.isfinite(Z).all()          # no self loops, distinct rows: FR's 1/s stays finite
 
 
+def _row_order(bits=32):
+    import ctypes as C
+    sc, lo, hi = C.c_int(), C.c_uint(), C.c_uint()
+    assert fa.load(bits).fusedMM_amd_last_row_order(C.byref(sc), C.byref(lo), C.byref(hi)) == 0
+    return sc.value, lo.value, hi.value
+
+
+@pytest.mark.parametrize("name,sd,scattered", [("c4", 6, 1), ("c3", 5, 1), ("c2", 3, 0), ("c5", 3, 0)])
+def test_row_order_follows_where_the_edges_are(oracle, name, sd, scattered):
+    """R-MAT degrees follow the bits of the row id, so one half of the row space holds far more
+    edges than the other: the row phase then takes stretches of 512 rows in scattered order.
+    Uniform and Zipf-random graphs keep the plain order.  Either way every row of Z equals the
+    oracle's, bit for bit: each row is one wavefront's work, whenever it is done."""
+    tkern, k, sk = _kind(name)
+    g, X, Y = bench.make_workload(name, sd)
+    assert g["rows"] >= 1 << 17                       # enough chunks for dynamic claims and many stretches
+    gpu_api.set_kind(sk, 32)
+    Z0 = np.zeros((g["rows"], k), np.float32)
+    rc, Z = gpu_api.run(MSG[tkern], g, X, Y, Z0, beta=0.0, bits=32)
+    assert rc == 0
+    sc, lo, hi = _row_order()
+    deg = np.diff(g["rowptr"]).astype(np.int64)
+    heavy_deg, seg_len = gpu_api.default_split(k)
+    light = np.where(deg <= heavy_deg, deg, 0)
+    half = g["rows"] // 2
+    true_ratio = light[:half].sum() / max(1, light[half:].sum())
+    print(name, "scattered", sc, "sampled", lo, hi, "true ratio of the halves %.3f" % true_ratio, flush=True)
+    assert sc == scattered
+    assert lo > 0 and hi > 0 and abs(lo / hi - true_ratio) < 0.25 * true_ratio      # the sample tells the truth
+    want = gpu_api.oracle_mirror(oracle, tkern, g, X, Y, Z0, 0.0, sk, k, heavy_deg, seg_len)
+    np.testing.assert_array_equal(Z.view(np.uint32), want.view(np.uint32))
+
+
 class Resident:
     """A workload uploaded once; calls go through the asynchronous entry point."""
 
