@@ -121,6 +121,7 @@ struct Globals {
    int seg_len = 0;
    int blocks_per_cu = 0;
    int validate = 0;
+   int row_order = 0;         // 0 auto, 1 first to last, 2 scattered stretches (FUSEDMM_ROW_ORDER)
    int cache = 0;             // 1: keep device mirrors of read-only host operands between calls
    unsigned long long cache_clock = 0;
    double phase_ms[3] = {0, 0, 0};   // upload, kernels, download of the last host-pointer call
@@ -160,6 +161,8 @@ void read_env_once()
    if (const char *e = getenv("FUSEDMM_BLOCKS_PER_CU")) g.blocks_per_cu = atoi(e);
    if (const char *e = getenv("FUSEDMM_VALIDATE")) g.validate = atoi(e);
    if (const char *e = getenv("FUSEDMM_CACHE")) g.cache = atoi(e) ? 1 : 0;
+   if (const char *e = getenv("FUSEDMM_ROW_ORDER"))   // "auto", "plain" (first to last) or "scattered"
+      g.row_order = !strcmp(e, "plain") ? 1 : (!strcmp(e, "scattered") ? 2 : 0);
    if (const char *e = getenv("FUSEDMM_SPLIT"))   // "heavy_deg,seg_len", as fusedMM_amd_set_split
    {
       long long h = 0;
@@ -550,6 +553,7 @@ int run_slab(const Args &a, const Plan &pl, int sop_kind, hipStream_t stream, in
    p.beta_zero = (pl.opt_rule && a.beta == 0.0f) ? 1 : 0;
    p.sop_kind = sop_kind;
    p.imessage = a.imessage;
+   p.row_order = g.row_order;
 
    // heavy-row split: segments of about 1 MiB of gathered rows but at most 2048 edges
    // (measured best on the R-MAT and power-law benchmark graphs: shorter segments pay

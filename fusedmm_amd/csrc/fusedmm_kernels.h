@@ -124,6 +124,7 @@ struct Params {
    unsigned int cap_heavy, cap_seg;
    int kpad;
    int row_counters;       // claim counters in use: kRowCounters; 1 when the grid has fewer waves; 0: wave w takes chunk w
+   int row_order;          // 0: decided from the classify kernel's sample; 1: first to last; 2: scattered stretches
 };
 
 // ---- wave primitives --------------------------------------------------------
@@ -887,7 +888,8 @@ __device__ __forceinline__ bool scattered_order(const Params<IdxT> &p)
    const int64_t nchunks = (p.m + kRowsPerClaim - 1) / kRowsPerClaim;
    const unsigned long long skew = p.ctr->skew;
    const unsigned long long e_lo = skew & 0xFFFFFFFFull, e_hi = skew >> 32;
-   return p.row_counters > 0 && (nchunks >> 6) > 1 && (4 * e_lo > 5 * e_hi || 4 * e_hi > 5 * e_lo);
+   if (p.row_counters <= 0 || (nchunks >> 6) <= 1 || p.row_order == 1) return false;
+   return p.row_order == 2 || 4 * e_lo > 5 * e_hi || 4 * e_hi > 5 * e_lo;
 }
 
 // Turn the value an atomicAdd on counter `cur` returned (in lane 0) into a

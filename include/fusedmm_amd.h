@@ -232,7 +232,8 @@ int fusedMM_amd_last_split(unsigned int *heavy_rows, unsigned int *segments, uns
  * more than 1.25 times the other (R-MAT graphs, vertices sorted by degree) and rows are claimed
  * dynamically, `scattered` is 1: the row phase then took stretches of 512 rows in a scattered order
  * instead of first to last, so that the GPU works on a mix of dense and sparse rows at any time.
- * Results do not depend on it.  Waits for the GPU. */
+ * Results do not depend on it.  The environment variable FUSEDMM_ROW_ORDER=plain | scattered | auto
+ * (read once, at the first call) overrides the choice.  Waits for the GPU. */
 int fusedMM_amd_last_row_order(int *scattered, unsigned int *edges_lower_half, unsigned int *edges_upper_half);
 
 /* Copy `bytes` (a multiple of 16, device memory, 16-byte aligned) with a plain
