@@ -42,3 +42,18 @@ def test_bench_line(flags, pipeline, bits, dtype):
     want = 262144 * (32 * vb + ib) + 16384 * ((3 if pipeline == "general" else 2) * 32 * vb + 2 * ib)
     assert rl["algorithmic_bytes"] == want
     assert rl["traffic"] is None                              # c1 is cache-resident: no counter traffic is quoted for it
+
+
+def test_forced_row_order_and_wide_z_rows_keep_the_bits():
+    """A uniform graph taken in scattered order (FUSEDMM_ROW_ORDER=scattered; the library would
+    not choose it here) with the rows of Z four times their length apart: the spot check
+    against the oracle still holds bit for bit, and the line says which order ran."""
+    env = dict(os.environ, FUSEDMM_ROW_ORDER="scattered")
+    r = subprocess.run([sys.executable, os.path.join(ROOT, "bench.py"), "--workload", "u512d64", "--steps", "2", "--warmup", "1",
+                        "--no-cpu", "--ldz", "2048"], stdout=subprocess.PIPE, stderr=subprocess.PIPE, text=True, timeout=170,
+                       env=env)
+    assert r.returncode == 0, r.stderr[-2000:]
+    out = json.loads(r.stdout.strip().splitlines()[-1])
+    assert out["spot_check_vs_oracle"] is True and out["row_order"]["scattered"] is True and out["config"]["ldz"] == 2048
+    lo, hi = out["row_order"]["sampled_edges_lower_half"], out["row_order"]["sampled_edges_upper_half"]
+    assert lo > 0 and abs(lo - hi) <= 0.05 * lo              # the sample itself says: evenly spread
