@@ -57,3 +57,19 @@ def test_traffic_figures_come_from_the_committed_profiles():
         assert 0.8 < got / 1e9 / float(m.group(2)) < 1.1, (w, got)
         assert "rocprofv3 --kernel-trace --stats" in text and "python3 bench.py --workload " + w in text
     assert bench.measured_traffic_bytes("c1") == (None, None)      # cache-resident case: no roofline claim
+
+
+def test_uniform_degree_workloads_and_the_bytes_of_the_general_rule():
+    sys.path.insert(0, ROOT)
+    import bench
+    from fusedmm_amd import synth
+    g, X, Y = bench.make_workload("u512d16", 8)
+    assert g["rows"] == 8192 and g["cols"] == 8192 and g["nnz"] == 8192 * 16 and X.shape == (8192, 512) and Y.shape == (8192, 512)
+    assert (np.diff(g["rowptr"]) == 16).all() and g["indx"].min() >= 0 and g["indx"].max() < 8192
+    g, X, Y = bench.make_workload("u512d512", 8)
+    assert g["rows"] == (1 << 17) // 512 and X.shape[0] == g["rows"] and Y.shape[0] == 8192      # fewer rows than columns
+    # the general rule reads Z before it writes it: one more row of K values per row; int64 indices: 8 bytes each
+    base = synth.algorithmic_bytes("s", 1000, 128, 16000, 4)
+    assert synth.algorithmic_bytes("s", 1000, 128, 16000, 4, beta_nonzero=True) == base + 1000 * 128 * 4
+    assert synth.algorithmic_bytes("s", 1000, 128, 16000, 8) == base + 16000 * 4 + 1000 * 2 * 4
+    assert synth.algorithmic_bytes("s", 1000, 128, 16000, 4, value_bytes=8) == 16000 * (1024 + 4) + 1000 * (2048 + 8)
