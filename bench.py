@@ -22,10 +22,18 @@ sys.path.insert(0, ROOT)
 
 PEAK_HBM_GBPS = 8000.0
 
-# HBM bytes per call from rocprofv3 --pmc FETCH_SIZE and WRITE_SIZE, each scaled by
-# the same counter's reading for a plain 1 GiB copy: measured, not computed, and
-# kept in the rocprofv3 summary of each workload under profiles/ (the line
-# "traffic_bytes_per_call: N"), where this reads it.
+# Bytes per call that crossed the L2 <-> data-fabric boundary, from rocprofv3 --pmc
+# FETCH_SIZE and WRITE_SIZE, each scaled by the same counter's reading for a plain
+# 1 GiB copy: measured, not computed, and kept in the rocprofv3 summary of each
+# workload under profiles/ (the line "traffic_bytes_per_call: N"), where this reads it.
+# These counters sit at the L2: what they count is served by HBM or by the 256 MiB
+# last-level (Infinity) cache behind the fabric, so on a workload whose Y partly fits
+# that cache (c2: 512 MiB) the figure is an upper bound on HBM bytes, not HBM bytes.
+TRAFFIC_IS = ("L2-miss (fabric) bytes per call: FETCH_SIZE + WRITE_SIZE scaled by a 1 GiB copy; served by HBM or by the "
+              "256 MiB last-level cache, so an upper bound on HBM bytes")
+# Extra workloads of the default run, measured after the headline one and reported under "also":
+# the second configuration with a bandwidth target (gcn K=256), then the skewed ones.
+ALSO_DEFAULT = ("c3g", "c3", "c4", "c5")   # c3g and c3 share a graph
 PROFILE_OF = {"c2": "fused_kernel_sigmoid_k128_c2.md", "c3": "spmm_k256_c3_rmat22.md",
               "c3g": "gcn_k256_c3g_rmat22.md", "c4": "tdist_k64_c4_rmat24.md", "c5": "sigmoid_k512_c5_zipf.md"}
 
@@ -51,6 +59,10 @@ WORKLOADS = {
     "c4g": ("gcn K=64 on the c4 graph (same gathers, no reduction or scalar op)", "g", 64, None),
     "c5": ("sigmoid K=512, Zipf(1.8) degrees n=2^21 nnz~4e7, hubs to 1e6", "s", 512, "sigmoid"),
 }
+# Narrow rows at HBM scale (the reference's own sweep is K = 32 ... 256): t-dist over an ER graph of 2^23
+# nodes with 2^27 edges, Y of 1 GiB (K=32) and 2 GiB (K=64): nothing fits a cache, rows are 128 and 256 bytes.
+WORKLOADS["k32er"] = ("tdist K=32, ER n=2^23 nnz=2^27 (128-byte rows, Y of 1 GiB)", "t", 32, "tdist")
+WORKLOADS["k64er"] = ("tdist K=64, ER n=2^23 nnz=2^27 (256-byte rows, Y of 2 GiB)", "t", 64, "tdist")
 # What a row length costs: sigmoid K=512 over a Y of 2^21 rows (c5's), every row with the
 # same number of uniformly random neighbours, min(2^21, 2^25 / degree) rows.
 for _d in (1, 4, 16, 64, 512):
@@ -84,6 +96,11 @@ def make_workload(name, scale_down=0):
         n = (1 << 21) >> sd
         g = synth.zipf_graph(n, 1.8, min(1000000, n // 2), 40000000 >> sd, 5)
         return g, synth.uniform_matrix(n, 512, -0.5, 0.5, 5, 1), synth.uniform_matrix(n, 512, -0.5, 0.5, 5, 2)
+    if name in ("k32er", "k64er"):
+        n = (1 << 23) >> sd
+        k = 32 if name == "k32er" else 64
+        g = synth.er_graph(n, 8 * n, 7)
+        return g, synth.uniform_matrix(n, k, -1.0, 1.0, 7, 1), synth.uniform_matrix(n, k, -1.0, 1.0, 7, 2)
     if name.startswith("u512d"):
         d = int(name[5:])
         n = (1 << 21) >> sd
@@ -176,14 +193,21 @@ def cpu_baseline(name, g, X, Y, tkern, kind_id, k, budget_s=12.0):
     return out
 
 
-def main():
+def parse_args(argv=None):
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--workload", default="c2", choices=sorted(WORKLOADS),
                     help="c1-c5: the benchmark configurations (c2 is the one the metric is quoted on); c3g, c4g: the gcn "
-                         "tuple on the c3 and c4 graphs; u512d<D>: uniform-degree rows at c5's row size (a measuring aid)")
+                         "tuple on the c3 and c4 graphs; k32er, k64er: narrow rows at HBM scale; u512d<D>: uniform-degree "
+                         "rows at c5's row size (a measuring aid)")
+    ap.add_argument("--also", default="auto",
+                    help="comma-separated workloads measured after the headline one and reported, compactly, under "
+                         "\"also\" in the same JSON line (each with its own roofline figures and spot check); 'auto' = "
+                         + ",".join(ALSO_DEFAULT) + " for the default run (c2, float, int32, optimised kernels), none "
+                         "otherwise; 'none' switches it off")
+    ap.add_argument("--also-steps", type=int, default=10, help="timed steps of each extra workload (2 warm-up steps)")
     ap.add_argument("--dtype", default="f32", choices=["f32", "f64"],
                     help="f64 runs the double-precision library (the reference's -DDREAL build)")
     ap.add_argument("--index-bits", type=int, default=32, choices=[32, 64],
@@ -200,41 +224,156 @@ def main():
                          "two kernels keeps them from being dispatched back to back, about 20 us per step, so the "
                          "timed region samples rather than instruments every step")
     ap.add_argument("--read-probe", action="store_true",
-                    help="also time a read-only stream over 4 GiB (what HBM delivers to reads alone) and report it")
+                    help="also time a read-only stream over 4 GiB (what the memory system delivers to reads alone) and report it")
     ap.add_argument("--ldz", type=int, default=0,
                     help="leading dimension of Z in elements (default K): rows of Z further apart in memory")
     ap.add_argument("--gather-probe", action="store_true",
-                    help="also time a read-only gather of uniformly random rows of the workload's row size from a buffer "
-                         "the size of its Y (what the memory system delivers to such gathers alone) and report it")
-    args = ap.parse_args()
-    if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
-        print("bench.py: this path is built and measured on ONE GPU; --gpus %d is not supported "
-              "(rows are independent: a sharded run would split the rows of A, X and Z across GPUs)" % args.gpus, file=sys.stderr)
-        sys.exit(2)
+                    help="time a read-only gather of uniformly random rows of the workload's row size from a buffer "
+                         "the size of its Y (what the memory system delivers to such gathers alone) and report it; "
+                         "always on for the default run and its extra workloads")
+    return ap.parse_args(argv)
 
-    import torch
-    import fusedmm_amd as fa
+
+def run_gather_probe(torch, probes, n, row_bytes, stream):
+    """Read-only gather of 4 GiB of uniformly random rows of row_bytes out of a buffer of n rows."""
+    dev = torch.device("cuda:0")
+    nbytes = n * row_bytes
+    src = torch.empty(nbytes // 4, dtype=torch.float32, device=dev).uniform_(-1, 1)
+    sink = torch.zeros(4, dtype=torch.int32, device=dev)
+    n_ids = (4 << 30) // row_bytes
+    gen = torch.Generator(device=dev)
+    gen.manual_seed(11)
+    ids = torch.randint(0, n, (n_ids,), device=dev, dtype=torch.int64, generator=gen).to(torch.int32)
+    out = {"row_bytes": row_bytes, "buffer_bytes": nbytes, "gathered_bytes": n_ids * row_bytes}
+    for label, nt in (("plain_loads", 0), ("nontemporal_loads", 1)):
+        launch = lambda: probes.fusedMM_amd_gather_probe(src.data_ptr(), row_bytes, ids.data_ptr(), n_ids, 4, 8, nt,
+                                                         sink.data_ptr(), stream)
+        for _ in range(2):
+            assert launch() == 0
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(10):
+            launch()
+        e1.record()
+        torch.cuda.synchronize()
+        out[label + "_GBps"] = n_ids * row_bytes / (e0.elapsed_time(e1) / 10 * 1e-3) / 1e9
+    del src, sink, ids
+    return out
+
+
+def run_read_probe(torch, probes, stream):
+    dev = torch.device("cuda:0")
+    nbytes = 4 << 30
+    src = torch.empty(nbytes // 4, dtype=torch.float32, device=dev).uniform_(-1, 1)
+    sink = torch.zeros(4, dtype=torch.int32, device=dev)
+    out = {"bytes": nbytes}
+    for label, nt in (("plain_loads", 0), ("nontemporal_loads", 1)):
+        for _ in range(2):
+            assert probes.fusedMM_amd_read_probe(src.data_ptr(), nbytes, 16, 8, nt, sink.data_ptr(), stream) == 0
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(10):
+            probes.fusedMM_amd_read_probe(src.data_ptr(), nbytes, 16, 8, nt, sink.data_ptr(), stream)
+        e1.record()
+        torch.cuda.synchronize()
+        out[label + "_GBps"] = nbytes / (e0.elapsed_time(e1) / 10 * 1e-3) / 1e9
+    del src, sink
+    return out
+
+
+_graphs = {}
+
+
+def workload_data(name):
+    """make_workload(), the graph shared by workloads that differ in the op tuple only (c3/c3g, c4/c4g)."""
+    key = {"c3g": "c3", "c4g": "c4"}.get(name, name)
+    if key not in _graphs:
+        _graphs.clear()                     # one graph at a time: the large ones take several GB of host memory
+        _graphs[key] = make_workload(key)
+    return _graphs[key]
+
+
+def spot_check(torch, name, g, X, Y, d_Z, k, ldz, tkern, kind_id, vbits, general, step):
+    """A window of rows from the middle of the matrix plus the longest row, against the oracle (checker only):
+    bit for bit for the optimised kernels, to the parity tests' tolerance for the general pipeline."""
+    m = g["rows"]
+    np_v = np.float32 if vbits == 32 else np.float64
+    if general:
+        # the general rule folded every step into Z; one more step on a cleared Z is
+        # what the oracle (Z0 = 0) is compared with
+        d_Z.zero_()
+        step()
+        torch.cuda.synchronize()
+    sys.path.insert(0, os.path.join(ROOT, "tests"))
+    from oracle_api import Oracle
+    from gpu_api import oracle_mirror, default_split
+    orc = Oracle(vbits=vbits)
+    heavy_deg, seg_len = default_split(k, vbits)
+    deg = np.diff(g["rowptr"])
+    windows = [(m // 2, min(m, m // 2 + 1024))]
+    hub = int(np.argmax(deg))
+    # (the general pipeline's tolerance check holds a row's terms in double precision: rows to 10^5 edges)
+    if deg[hub] <= (100000 if general else 1200000):
+        windows.append((hub, hub + 1))
+    ok = True
+    for lo, hi in windows:
+        sub = dict(g)
+        sub.update(rows=hi - lo, pntrb=g["pntrb"][lo:hi], pntre=g["pntre"][lo:hi])
+        Xs = None if X is None else X[lo:hi]
+        want = oracle_mirror(orc, tkern, sub, Xs, Y, np.zeros((hi - lo, k), np_v), 0.0, kind_id, k, heavy_deg, seg_len)
+        got = np.ascontiguousarray(d_Z[lo:hi, :k].cpu().numpy())
+        if not general:
+            ok = ok and bool(np.array_equal(got.view(np.uint8), want.view(np.uint8)))
+            continue
+        # The general pipeline multiplies and adds where the optimised kernels fuse, so
+        # its bits differ from the mirror's: it is held to the tolerance of the parity
+        # tests against the oracle's double-precision evaluation instead.
+        import checks
+        ot = "t" if tkern == "f" else tkern
+        z64 = np.zeros((hi - lo, k), np_v)
+        es = np.zeros(int(sub["pntre"].max()) if hi > lo else 0, np_v)
+        orc.opt(ot, sub, Xs, Y, z64, beta=0.0, sop_kind=kind_id, mode=1, edge_s=es if kind_id else None)
+        _, slots = checks.edge_rows(sub)
+        d_abs = (np.ones(slots.size) if tkern == "g" else np.abs(g["val"][slots]).astype(np.float64) if tkern == "m"
+                 else np.abs(orc.sop(kind_id, es[slots])).astype(np.float64))
+        sdeg = (sub["pntre"] - sub["pntrb"]).astype(np.int64)
+        extra = 4 * checks.EPS32 * np.sqrt(np.maximum(sdeg, 1))[:, None] * checks.abs_term_sum(tkern, sub, Xs, Y, d_abs)
+        if tkern == "s":
+            extra = extra + checks.sigmoid_flip_slack(orc.table(), sub, Xs, Y)[0]
+        rtol = 1e-5 if tkern in ("g", "m") else 1e-4
+        try:
+            checks.assert_close(got, z64, rtol, 1e-6, extra, "general pipeline, rows %d..%d" % (lo, hi))
+        except AssertionError as e:
+            print("bench.py: %s: %s" % (name, e), file=sys.stderr)
+            ok = False
+    return ok
+
+
+def measure(torch, fa, probes, name, steps, warmup, args, gather_probe, read_probe=False, copy_probe=False):
+    """Time `steps` calls of fusedMM_csr_stream on workload `name`, operands resident.  Returns the figures of the
+    JSON line for that workload and what the CPU leg needs (graph, embeddings)."""
     from fusedmm_amd import synth
-
-    desc, tkern, k, kind = WORKLOADS[args.workload]
+    desc, tkern, k, kind = WORKLOADS[name]
     bits = args.index_bits
     vbits = 32 if args.dtype == "f32" else 64
     np_v = np.float32 if vbits == 32 else np.float64
     lib = fa.load(bits, vbits)
     kind_id = {None: 0, "sigmoid": 1, "tdist": 2, "fr": 3}[kind]
     lib.fusedMM_amd_set_sop_kind(kind_id)
-    if args.general:
-        lib.fusedMM_amd_set_opt(0)
+    lib.fusedMM_amd_set_opt(0 if args.general else 1)
     imsg = {"s": fa.MSG_SIGMOID, "t": fa.MSG_TDIST, "f": fa.MSG_FR, "m": fa.MSG_SPMM, "g": fa.MSG_GCN}[tkern]
 
     t_gen = time.time()
-    g, X, Y = make_workload(args.workload)
+    g, X, Y = workload_data(name)
     if vbits == 64:
         same = Y is X
         X = None if X is None else X.astype(np_v)
         Y = X if same else Y.astype(np_v)
-        g["val"] = g["val"].astype(np_v)
+        g = dict(g, val=g["val"].astype(np_v))
     if bits == 64:
+        g = dict(g)
         for key in ("indx", "pntrb", "pntre", "rowptr"):
             g[key] = g[key].astype(np.int64)
     t_gen = time.time() - t_gen
@@ -255,65 +394,26 @@ def main():
         if rc != 0:
             raise SystemExit("fusedMM_csr returned %d" % rc)
 
-    if args.copy_probe:
+    if copy_probe:
         src = torch.ones(1 << 28, dtype=torch.float32, device=dev)
         dst = torch.empty_like(src)
         for _ in range(3):
-            assert lib.fusedMM_amd_copy_probe(dst.data_ptr(), src.data_ptr(), 1 << 30, stream) == 0
+            assert probes.fusedMM_amd_copy_probe(dst.data_ptr(), src.data_ptr(), 1 << 30, stream) == 0
         torch.cuda.synchronize()
         del src, dst
 
-    read_probe = None
-    if args.read_probe:
-        nbytes = 4 << 30
-        src = torch.empty(nbytes // 4, dtype=torch.float32, device=dev).uniform_(-1, 1)
-        sink = torch.zeros(4, dtype=torch.int32, device=dev)
-        read_probe = {"bytes": nbytes}
-        for label, nt in (("plain_loads", 0), ("nontemporal_loads", 1)):
-            for _ in range(2):
-                assert lib.fusedMM_amd_read_probe(src.data_ptr(), nbytes, 16, 8, nt, sink.data_ptr(), stream) == 0
-            torch.cuda.synchronize()
-            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-            e0.record()
-            for _ in range(10):
-                lib.fusedMM_amd_read_probe(src.data_ptr(), nbytes, 16, 8, nt, sink.data_ptr(), stream)
-            e1.record()
-            torch.cuda.synchronize()
-            read_probe[label + "_GBps"] = nbytes / (e0.elapsed_time(e1) / 10 * 1e-3) / 1e9
-        del src, sink
-
-    gather_probe = None
+    rp = run_read_probe(torch, probes, stream) if read_probe else None
+    gp = None
     row_bytes = k * (vbits // 8)
-    if args.gather_probe and row_bytes <= 2048 and (row_bytes & (row_bytes - 1)) == 0 and row_bytes >= 16:
-        nbytes = n * row_bytes
-        src = torch.empty(nbytes // 4, dtype=torch.float32, device=dev).uniform_(-1, 1)
-        sink = torch.zeros(4, dtype=torch.int32, device=dev)
-        n_ids = (4 << 30) // row_bytes                       # 4 GiB gathered per launch
-        gen = torch.Generator(device=dev)
-        gen.manual_seed(11)
-        ids = torch.randint(0, n, (n_ids,), device=dev, dtype=torch.int64, generator=gen).to(torch.int32)
-        gather_probe = {"row_bytes": row_bytes, "buffer_bytes": nbytes, "gathered_bytes": n_ids * row_bytes}
-        for label, nt in (("plain_loads", 0), ("nontemporal_loads", 1)):
-            launch = lambda: lib.fusedMM_amd_gather_probe(src.data_ptr(), row_bytes, ids.data_ptr(), n_ids, 4, 8, nt,
-                                                          sink.data_ptr(), stream)
-            for _ in range(2):
-                assert launch() == 0
-            torch.cuda.synchronize()
-            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-            e0.record()
-            for _ in range(10):
-                launch()
-            e1.record()
-            torch.cuda.synchronize()
-            gather_probe[label + "_GBps"] = n_ids * row_bytes / (e0.elapsed_time(e1) / 10 * 1e-3) / 1e9
-        del src, sink, ids
+    if gather_probe and 16 <= row_bytes <= 2048 and (row_bytes & (row_bytes - 1)) == 0:
+        gp = run_gather_probe(torch, probes, n, row_bytes, stream)
 
-    for _ in range(args.warmup):
+    for _ in range(warmup):
         step()
     torch.cuda.synchronize()
     lib.fusedMM_amd_timing(max(0, args.kernel_events_every))
     t0 = time.perf_counter()
-    for _ in range(args.steps):
+    for _ in range(steps):
         step()
     torch.cuda.synchronize()
     wall = time.perf_counter() - t0
@@ -325,7 +425,7 @@ def main():
         if lib.fusedMM_amd_timing_call(i, C.byref(c_), C.byref(f_), C.byref(m_)) == 0:
             per_call.append(c_.value + f_.value + m_.value)
     lib.fusedMM_amd_timing(0)
-    ms_per_step = wall / args.steps * 1e3
+    ms_per_step = wall / steps * 1e3
 
     flops = synth.algorithmic_flops(tkern, k, nnz)
     # the general rule reads Z before it writes it
@@ -348,82 +448,26 @@ def main():
         dom_ms = ms_per_step      # no step carried events: whole-step wall time stands in (an upper bound)
     achieved = b_alg / (dom_ms * 1e-3) / 1e9 if dom_ms > 0 else 0.0
     as_profiled = vbits == 32 and bits == 32 and not args.general
-    traffic, traffic_from = measured_traffic_bytes(args.workload) if as_profiled else (None, None)
+    traffic, traffic_from = measured_traffic_bytes(name) if as_profiled else (None, None)
     roofline = {"bound": "hbm", "achieved": achieved, "peak": PEAK_HBM_GBPS, "unit": "GB/s",
                 "frac": achieved / PEAK_HBM_GBPS, "traffic": traffic, "traffic_from": traffic_from,
+                "traffic_is": TRAFFIC_IS if traffic else None,
                 "kernel": "classify_kernel+fused_kernel+merge_kernel" if split else "fused_kernel",
                 "kernel_ms": dom_ms, "algorithmic_bytes": b_alg}
-    if read_probe:
-        roofline["read_stream_probe"] = read_probe
-        roofline["frac_of_read_stream"] = achieved / read_probe["plain_loads_GBps"]
-
-    if gather_probe:
-        roofline["gather_probe"] = gather_probe
-        roofline["frac_of_gather_probe"] = achieved / gather_probe["plain_loads_GBps"]
+    if rp:
+        roofline["read_stream_probe"] = rp
+        roofline["frac_of_read_stream"] = achieved / rp["plain_loads_GBps"]
+    if gp:
+        roofline["gather_probe"] = gp
+        roofline["frac_of_gather_probe"] = achieved / gp["plain_loads_GBps"]
 
     checked = None
     if not args.no_check:
-        if args.general:
-            # the general rule folded every step into Z; one more step on a cleared Z is
-            # what the oracle (Z0 = 0) is compared with
-            d_Z.zero_()
-            step()
-            torch.cuda.synchronize()
-        # Spot check against the oracle (checker only), bit for bit: a window of
-        # rows from the middle of the matrix plus the longest row, passed to the
-        # oracle as sub-problems (row pointers and X offset to the window).
-        sys.path.insert(0, os.path.join(ROOT, "tests"))
-        from oracle_api import Oracle
-        from gpu_api import oracle_mirror, default_split
-        orc = Oracle(vbits=vbits)
-        heavy_deg, seg_len = default_split(k, vbits)
-        deg = np.diff(g["rowptr"])
-        windows = [(m // 2, min(m, m // 2 + 1024))]
-        hub = int(np.argmax(deg))
-        # (the general pipeline's tolerance check holds a row's terms in double precision: rows to 10^5 edges)
-        if deg[hub] <= (100000 if args.general else 1200000):
-            windows.append((hub, hub + 1))
-        z_all = d_Z[:, :k].cpu().numpy() if m * ldz <= (1 << 28) else None
-        checked = True
-        for lo, hi in windows:
-            sub = dict(g)
-            sub.update(rows=hi - lo, pntrb=g["pntrb"][lo:hi], pntre=g["pntre"][lo:hi])
-            Xs = None if X is None else X[lo:hi]
-            want = oracle_mirror(orc, tkern, sub, Xs, Y, np.zeros((hi - lo, k), np_v), 0.0, kind_id, k,
-                                 heavy_deg, seg_len)
-            got = z_all[lo:hi] if z_all is not None else d_Z[lo:hi, :k].cpu().numpy()
-            got = np.ascontiguousarray(got)
-            if not args.general:
-                checked = checked and bool(np.array_equal(got.view(np.uint8), want.view(np.uint8)))
-                continue
-            # The general pipeline multiplies and adds where the optimised kernels fuse, so
-            # its bits differ from the mirror's: it is held to the tolerance of the parity
-            # tests against the oracle's double-precision evaluation instead.
-            import checks
-            ot = "t" if tkern == "f" else tkern
-            z64 = np.zeros((hi - lo, k), np_v)
-            es = np.zeros(int(sub["pntre"].max()) if hi > lo else 0, np_v)
-            orc.opt(ot, sub, Xs, Y, z64, beta=0.0, sop_kind=kind_id, mode=1, edge_s=es if kind_id else None)
-            _, slots = checks.edge_rows(sub)
-            d_abs = (np.ones(slots.size) if tkern == "g" else np.abs(g["val"][slots]).astype(np.float64) if tkern == "m"
-                     else np.abs(orc.sop(kind_id, es[slots])).astype(np.float64))
-            sdeg = (sub["pntre"] - sub["pntrb"]).astype(np.int64)
-            extra = 4 * checks.EPS32 * np.sqrt(np.maximum(sdeg, 1))[:, None] * checks.abs_term_sum(tkern, sub, Xs, Y, d_abs)
-            if tkern == "s":
-                extra = extra + checks.sigmoid_flip_slack(orc.table(), sub, Xs, Y)[0]
-            rtol = 1e-5 if tkern in ("g", "m") else 1e-4
-            try:
-                checks.assert_close(got, z64, rtol, 1e-6, extra, "general pipeline, rows %d..%d" % (lo, hi))
-            except AssertionError as e:
-                print("bench.py: %s" % e, file=sys.stderr)
-                checked = False
+        checked = spot_check(torch, name, g, X, Y, d_Z, k, ldz, tkern, kind_id, vbits, args.general, step)
 
     out = {
-        "metric": "GFLOP/s + HBM GB/s (% of peak), sigmoid K=128, 1 MI355X vs CPU OpenMP",
-        "value": value, "unit": "GFLOP/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
-        "ms_per_step": ms_per_step, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
-        "dtype": args.dtype, "data": "synthetic",
-        "config": {"workload": "%s: %s" % (args.workload, desc), "op": tkern, "K": k, "rows": m, "nnz": nnz,
+        "value": value, "unit": "GFLOP/s", "steps": steps, "warmup": warmup, "ms_per_step": ms_per_step,
+        "config": {"workload": "%s: %s" % (name, desc), "op": tkern, "K": k, "rows": m, "nnz": nnz,
                    "index_bits": bits, "beta": 0.0, "graph_gen_s": round(t_gen, 2),
                    "pipeline": "general" if args.general else "optimised", "ldz": ldz},
         "edges_per_s": nnz / (ms_per_step * 1e-3),
@@ -438,12 +482,74 @@ def main():
         "spot_check_vs_oracle": checked,
         "roofline": roofline,
     }
+    del d_val, d_indx, d_pb, d_pe, d_X, d_Y, d_Z
+    torch.cuda.empty_cache()
+    return out, (g, X, Y, tkern, kind_id, k, as_profiled)
+
+
+def compact(name, r):
+    """What the "also" list keeps of an extra workload's figures."""
+    rl = r["roofline"]
+    return {"workload": r["config"]["workload"], "op": r["config"]["op"], "K": r["config"]["K"], "rows": r["config"]["rows"],
+            "nnz": r["config"]["nnz"], "steps": r["steps"], "warmup": r["warmup"], "ms_per_step": r["ms_per_step"],
+            "value": r["value"], "unit": r["unit"], "edges_per_s": r["edges_per_s"], "kernel_ms": rl["kernel_ms"],
+            "kernels": rl["kernel"], "algorithmic_bytes": rl["algorithmic_bytes"],
+            "roofline": {"bound": "hbm", "achieved": rl["achieved"], "peak": rl["peak"], "unit": rl["unit"],
+                         "frac": rl["frac"], "traffic": rl["traffic"], "traffic_from": rl["traffic_from"],
+                         "frac_of_gather_probe": rl.get("frac_of_gather_probe"),
+                         "gather_probe_GBps": (rl.get("gather_probe") or {}).get("plain_loads_GBps")},
+            "split": r["split"], "row_order_scattered": r["row_order"]["scattered"],
+            "graph_gen_s": r["config"]["graph_gen_s"], "spot_check_vs_oracle": r["spot_check_vs_oracle"]}
+
+
+def main():
+    args = parse_args()
+    if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
+        print("bench.py: this path is built and measured on ONE GPU; --gpus %d is not supported "
+              "(rows are independent: a sharded run would split the rows of A, X and Z across GPUs)" % args.gpus, file=sys.stderr)
+        sys.exit(2)
+
+    import torch
+    import fusedmm_amd as fa
+    probes = fa.load_probes()
+
+    default_run = (args.workload == "c2" and args.dtype == "f32" and args.index_bits == 32 and not args.general)
+    also_names = []
+    if args.also == "auto":
+        also_names = list(ALSO_DEFAULT) if default_run else []
+    elif args.also not in ("none", ""):
+        also_names = [w for w in args.also.split(",") if w]
+        for w in also_names:
+            if w not in WORKLOADS:
+                raise SystemExit("unknown workload %s in --also" % w)
+
+    r, (g, X, Y, tkern, kind_id, k, as_profiled) = measure(
+        torch, fa, probes, args.workload, args.steps, args.warmup, args,
+        gather_probe=args.gather_probe or default_run, read_probe=args.read_probe, copy_probe=args.copy_probe)
+    out = {"metric": "GFLOP/s + HBM GB/s (% of peak), sigmoid K=128, 1 MI355X vs CPU OpenMP",
+           "value": r["value"], "unit": r["unit"], "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+           "ms_per_step": r["ms_per_step"], "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+           "dtype": args.dtype, "data": "synthetic"}
+    for key in ("config", "edges_per_s", "hbm_GBps_algorithmic", "pct_peak_hbm", "kernel_ms", "kernel_events",
+                "kernels_ms_per_call", "split", "row_order", "spot_check_vs_oracle", "roofline"):
+        out[key] = r[key]
+    failed = [args.workload] if r["spot_check_vs_oracle"] is False else []
     if not args.no_cpu and as_profiled:
         out["cpu_baseline"] = cpu_baseline(args.workload, g, X, Y, tkern, kind_id, k)
-    if checked is False:
+    del g, X, Y
+
+    if also_names:
+        out["also"] = []
+        for w in also_names:
+            print("bench.py: extra workload %s ..." % w, file=sys.stderr, flush=True)
+            ra, _ = measure(torch, fa, probes, w, args.also_steps, 2, args, gather_probe=True)
+            out["also"].append(compact(w, ra))
+            if ra["spot_check_vs_oracle"] is False:
+                failed.append(w)
+    if failed:
         # a run whose output differs from the oracle's is not a measurement
         out["value"] = None
-        out["error"] = "spot check against the oracle failed: results differ"
+        out["error"] = "spot check against the oracle failed on %s: results differ" % ", ".join(failed)
         print(json.dumps(out))
         sys.exit(3)
     print(json.dumps(out))

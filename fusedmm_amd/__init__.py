@@ -114,6 +114,11 @@ def load(index_bits=32, value_bits=32):
     return lib
 
 
+def load_probes():
+    """The measuring aids (copy, read-stream and gather probes): bench.py's yardsticks, not part of the product ABI."""
+    return load(32, 32)
+
+
 def _addr(a):
     """Raw address of a numpy array, a torch tensor, an int, or None."""
     if a is None:

@@ -73,3 +73,40 @@ def test_uniform_degree_workloads_and_the_bytes_of_the_general_rule():
     assert synth.algorithmic_bytes("s", 1000, 128, 16000, 4, beta_nonzero=True) == base + 1000 * 128 * 4
     assert synth.algorithmic_bytes("s", 1000, 128, 16000, 8) == base + 16000 * 4 + 1000 * 2 * 4
     assert synth.algorithmic_bytes("s", 1000, 128, 16000, 4, value_bytes=8) == 16000 * (1024 + 4) + 1000 * (2048 + 8)
+
+
+def test_the_default_run_also_times_the_other_bandwidth_target_and_the_skewed_graphs():
+    """The one JSON line of the default run carries, under "also", the gcn K=256 configuration (the second one
+    with a bandwidth target) first, then the skewed graphs; each entry has its own roofline figures and spot check."""
+    sys.path.insert(0, ROOT)
+    import bench
+    assert bench.ALSO_DEFAULT[0] == "c3g" and set(bench.ALSO_DEFAULT) == {"c3g", "c4", "c5", "c3"}
+    assert all(w in bench.WORKLOADS and w in bench.PROFILE_OF for w in bench.ALSO_DEFAULT)
+    full = {"value": 1.0, "unit": "GFLOP/s", "steps": 10, "warmup": 2, "ms_per_step": 2.0, "edges_per_s": 3.0,
+            "config": {"workload": "c3g: x", "op": "g", "K": 256, "rows": 4, "nnz": 5, "graph_gen_s": 1.0},
+            "split": {"heavy_rows": 1, "segments": 2, "overflow": 0}, "row_order": {"scattered": True},
+            "spot_check_vs_oracle": True,
+            "roofline": {"bound": "hbm", "achieved": 6400.0, "peak": 8000.0, "unit": "GB/s", "frac": 0.8, "traffic": 7,
+                         "traffic_from": "profiles/x.md", "kernel": "fused_kernel", "kernel_ms": 1.9,
+                         "algorithmic_bytes": 11, "frac_of_gather_probe": 1.1, "gather_probe": {"plain_loads_GBps": 5800.0}}}
+    c = bench.compact("c3g", full)
+    for key in ("workload", "ms_per_step", "kernel_ms", "algorithmic_bytes", "roofline", "split", "spot_check_vs_oracle"):
+        assert key in c, key
+    assert c["roofline"]["frac"] == 0.8 and c["roofline"]["traffic"] == 7 and c["roofline"]["frac_of_gather_probe"] == 1.1
+    assert c["roofline"]["gather_probe_GBps"] == 5800.0 and c["kernel_ms"] == 1.9 and c["row_order_scattered"] is True
+    # the narrow-row workloads: 2^23 rows of 128 and 256 bytes, 2^27 edges
+    g, X, Y = bench.make_workload("k32er", 10)
+    assert g["rows"] == 8192 and g["nnz"] == 16 * 8192 and X.shape == (8192, 32) and X is not Y
+    assert bench.WORKLOADS["k64er"][2] == 64 and "L2-miss" in bench.TRAFFIC_IS
+
+
+def test_also_rejects_unknown_workloads_before_touching_the_gpu():
+    a = bench_args("--also", "c3g,c4")
+    assert a.also == "c3g,c4" and a.also_steps == 10
+    assert bench_args().also == "auto"
+
+
+def bench_args(*argv):
+    sys.path.insert(0, ROOT)
+    import bench
+    return bench.parse_args(list(argv))

@@ -57,3 +57,19 @@ def test_forced_row_order_and_wide_z_rows_keep_the_bits():
     assert out["spot_check_vs_oracle"] is True and out["row_order"]["scattered"] is True and out["config"]["ldz"] == 2048
     lo, hi = out["row_order"]["sampled_edges_lower_half"], out["row_order"]["sampled_edges_upper_half"]
     assert lo > 0 and abs(lo - hi) <= 0.05 * lo              # the sample itself says: evenly spread
+
+
+def test_extra_workloads_ride_in_the_same_line():
+    """--also: the extra workloads are measured after the headline one and reported compactly in the same
+    single JSON line, each with its own roofline figures, gather probe and spot check."""
+    out = _bench("--also", "c1,u512d64", "--also-steps", "2")
+    assert out["config"]["workload"].startswith("c1:") and "gather_probe" not in out["roofline"]
+    also = out["also"]
+    assert [a["workload"].split(":")[0] for a in also] == ["c1", "u512d64"]
+    for a in also:
+        assert a["spot_check_vs_oracle"] is True and a["steps"] == 2 and a["ms_per_step"] > 0 and a["kernel_ms"] > 0
+        rl = a["roofline"]
+        assert rl["bound"] == "hbm" and abs(rl["frac"] - rl["achieved"] / 8000.0) < 1e-12
+        assert rl["gather_probe_GBps"] > 0 and abs(rl["frac_of_gather_probe"] - rl["achieved"] / rl["gather_probe_GBps"]) < 1e-9
+        assert a["algorithmic_bytes"] > 0 and set(a["split"]) == {"heavy_rows", "segments", "overflow"}
+    assert also[0]["algorithmic_bytes"] == 262144 * 132 + 16384 * 264
