@@ -125,71 +125,89 @@ def physical_cores():
         return None
 
 
-def sample_rows(g, edge_budget):
-    """Leading rows of the graph holding about edge_budget edges (all rows when the graph is smaller)."""
+def sample_problem(g, X, edge_budget, seed=17):
+    """A sub-problem of about edge_budget edges for the CPU legs: the whole graph when it is that small, else rows
+    drawn uniformly at random (seeded) from all over the matrix, kept in ascending order, with their X rows; Y and
+    the CSR arrays are the workload's own (pntrb / pntre of the chosen rows: m < rows and separate row pointers are
+    part of the API).  Returns (graph dict, X, rows chosen or None)."""
     rows = g["rows"]
     if g["nnz"] <= edge_budget:
-        return rows
-    m = int(np.searchsorted(g["pntre"][:rows].astype(np.int64), edge_budget, side="right"))
-    return max(1, min(rows, m))
+        return g, X, None
+    deg = (g["pntre"][:rows].astype(np.int64) - g["pntrb"][:rows].astype(np.int64))
+    order = np.random.Generator(np.random.Philox(key=[seed, 0])).permutation(rows)
+    take = int(np.searchsorted(np.cumsum(deg[order]), edge_budget, side="right"))
+    pick = np.sort(order[:max(1, take)])
+    sub = dict(g)
+    sub.update(rows=int(pick.size), pntrb=np.ascontiguousarray(g["pntrb"][pick]), pntre=np.ascontiguousarray(g["pntre"][pick]))
+    sub.pop("rowptr", None)
+    return sub, (None if X is None else np.ascontiguousarray(X[pick])), pick
 
 
 def cpu_baseline(name, g, X, Y, tkern, kind_id, k, budget_s=12.0):
-    """The CPU oracle's OpenMP port timed on this host's cores, on a bounded
-    sample of the same workload: the leading rows of the graph (m < rows is part
-    of the API), all rows when that fits the time budget.  Next to it, on the same
-    sample, the real reference's general fusedMM_csr where oracle/_ref was built.
+    """The CPU legs, timed on this host's cores on a bounded sample of the same workload (sample_problem):
+    the oracle's OpenMP port of the optimised semantics (the headline CPU figure), and beside it the real
+    reference's general fusedMM_csr where oracle/_ref was built, both on the same number of threads.
     Checker-side code: used here only to report a baseline."""
     sys.path.insert(0, os.path.join(ROOT, "tests"))
-    from oracle_api import Oracle, Ref, ref_available
+    from oracle_api import Oracle, Ref, ref_available, ref_threads_for
     from fusedmm_amd import synth
     orc = Oracle(fast=True)
+    cores = physical_cores()
+    # the threads this process may use: OpenMP's own limit (OMP_NUM_THREADS, cgroup share), not above the physical cores
     threads = orc.max_threads()
+    if cores:
+        threads = max(1, min(threads, cores))
     rows = g["rows"]
     # about 5e7 edges/s on 8 cores at K=128: size the sample for a few calls inside the budget
-    m = sample_rows(g, int(2.5e9 / k))
-    nnz_s = int(g["pntre"][m - 1]) - int(g["pntrb"][0])
+    gs, Xs, pick = sample_problem(g, X, int(2.5e9 / k))
+    m = gs["rows"]
+    nnz_s = int((gs["pntre"][:m].astype(np.int64) - gs["pntrb"][:m].astype(np.int64)).sum())
     Z = np.zeros((m, k), np.float32)
     ot = "t" if tkern == "f" else tkern
-    orc.baseline(ot, g, X, Y, Z, 0.0, kind_id, threads, m=m)  # warm-up, untimed
+    orc.baseline(ot, gs, Xs, Y, Z, 0.0, kind_id, threads, m=m)  # warm-up, untimed
     t_all = []
     t0 = time.time()
     while (len(t_all) < 3 or time.time() - t0 < budget_s) and len(t_all) < 200:
         t1 = time.time()
-        orc.baseline(ot, g, X, Y, Z, 0.0, kind_id, threads, m=m)
+        orc.baseline(ot, gs, Xs, Y, Z, 0.0, kind_id, threads, m=m)
         t_all.append(time.time() - t1)
-    t = float(np.mean(t_all))
+    t, t_min = float(np.mean(t_all)), float(np.min(t_all))
     flops = synth.algorithmic_flops(tkern, k, nnz_s)
+    what = ("the whole graph" if pick is None else
+            "%d of %d rows drawn uniformly at random from the whole matrix (seed 17), in ascending order" % (m, rows))
     out = {"value": flops / t / 1e9, "unit": "GFLOP/s", "cores": threads, "kind": "port",
-           "sample": "first %d of %d rows of the same workload (%d of %d edges), %d calls, mean %.4f s/call; "
-                     "OpenMP restatement built -O3 -march=x86-64-v3 (AVX2+FMA, not the host's widest ISA)"
-                     % (m, rows, nnz_s, g["nnz"], len(t_all), t),
-           "omp_max_threads": threads, "lscpu_physical_cores": physical_cores(),
+           "value_best_call": flops / t_min / 1e9,
+           "sample": "%s: %d of %d edges, %d calls, mean %.4f s/call, min %.4f; OpenMP restatement of the optimised "
+                     "semantics built -O3 -march=%s" % (what, nnz_s, g["nnz"], len(t_all), t, t_min, orc.isa),
+           "omp_max_threads": orc.max_threads(), "lscpu_physical_cores": cores,
+           "s_per_call": {"mean": t, "min": t_min},
            "edges_per_s": nnz_s / t,
            "alg_GBps": synth.algorithmic_bytes(tkern, m, k, nnz_s) / t / 1e9}
-    # the real reference's general pipeline (fusedMM.c compiled where it lies, 8 OpenMP threads as its
-    # build fixes them) on the same rows: lets a reader relate the port to the reference on this host
+    # the real reference's general pipeline (fusedMM.c compiled where it lies; its build bakes the OpenMP team size
+    # in, so the library built for the thread count used above is loaded) on the same sample
     ref_kind = {"s": "sigmoid", "t": "tdist", "f": "fr", "m": "spmm", "g": "gcn"}[tkern]
-    if ref_available(ref_kind, 32, 32):
+    ref_threads = ref_threads_for(threads)
+    if ref_available(ref_kind, 32, 32, ref_threads):
         from oracle_api import MSG
-        ref = Ref(ref_kind, 32, 32)
+        ref = Ref(ref_kind, 32, 32, ref_threads)
         Zr = np.zeros((m, k), np.float32)
-        Xr = X if X is not None else Y
-        ref.fusedMM_csr(MSG[tkern], g, Xr, Y, Zr, 0.0, m=m)       # warm-up
+        Xr = Xs if Xs is not None else Y
+        ref.fusedMM_csr(MSG[tkern], gs, Xr, Y, Zr, 0.0, m=m)       # warm-up
         tr = []
         t0 = time.time()
         while (len(tr) < 2 or time.time() - t0 < 0.6 * budget_s) and len(tr) < 50:
             Zr[:] = 0
             t1 = time.time()
-            ref.fusedMM_csr(MSG[tkern], g, Xr, Y, Zr, 0.0, m=m)
+            ref.fusedMM_csr(MSG[tkern], gs, Xr, Y, Zr, 0.0, m=m)
             tr.append(time.time() - t1)
-        tm = float(np.mean(tr))
+        tm, tmin = float(np.mean(tr)), float(np.min(tr))
         out["reference_general"] = {"kind": "reference-general", "value": flops / tm / 1e9, "unit": "GFLOP/s",
-                                    "cores": 8, "edges_per_s": nnz_s / tm,
-                                    "sample": "same rows; the reference's general fusedMM_csr (five indirect stage calls "
-                                              "per edge, NTHREADS=8 fixed at build time), %d calls, mean %.4f s/call; "
-                                              "its optimised kernels need its code generator and are not built here"
-                                              % (len(tr), tm)}
+                                    "value_best_call": flops / tmin / 1e9,
+                                    "cores": ref_threads, "edges_per_s": nnz_s / tm, "s_per_call": {"mean": tm, "min": tmin},
+                                    "sample": "same sample; the reference's general fusedMM_csr (five indirect stage calls "
+                                              "per edge, built -fopenmp -O3 with NTHREADS=%d), %d calls, mean %.4f s/call, "
+                                              "min %.4f; its optimised kernels are generated code and are not built here"
+                                              % (ref_threads, len(tr), tm, tmin)}
     return out
 
 
@@ -308,9 +326,11 @@ def spot_check(torch, name, g, X, Y, d_Z, k, ldz, tkern, kind_id, vbits, general
         torch.cuda.synchronize()
     sys.path.insert(0, os.path.join(ROOT, "tests"))
     from oracle_api import Oracle
-    from gpu_api import oracle_mirror, default_split
+    from gpu_api import oracle_mirror, default_split, packed_rows
     orc = Oracle(vbits=vbits)
     heavy_deg, seg_len = default_split(k, vbits)
+    # which rows were walked one per sub-wave: decided on groups of rows of the whole matrix (FUSEDMM_PACK_ROWS=off: none)
+    packed_all = packed_rows(g, m, k, vbits, heavy_deg, pack=os.environ.get("FUSEDMM_PACK_ROWS", "auto") != "off")
     deg = np.diff(g["rowptr"])
     windows = [(m // 2, min(m, m // 2 + 1024))]
     hub = int(np.argmax(deg))
@@ -322,7 +342,8 @@ def spot_check(torch, name, g, X, Y, d_Z, k, ldz, tkern, kind_id, vbits, general
         sub = dict(g)
         sub.update(rows=hi - lo, pntrb=g["pntrb"][lo:hi], pntre=g["pntre"][lo:hi])
         Xs = None if X is None else X[lo:hi]
-        want = oracle_mirror(orc, tkern, sub, Xs, Y, np.zeros((hi - lo, k), np_v), 0.0, kind_id, k, heavy_deg, seg_len)
+        want = oracle_mirror(orc, tkern, sub, Xs, Y, np.zeros((hi - lo, k), np_v), 0.0, kind_id, k, heavy_deg, seg_len,
+                             packed=packed_all[lo:hi])
         got = np.ascontiguousarray(d_Z[lo:hi, :k].cpu().numpy())
         if not general:
             ok = ok and bool(np.array_equal(got.view(np.uint8), want.view(np.uint8)))

@@ -8,7 +8,7 @@ load time, a failing call returns the library's status code.
 import ctypes as C
 import os
 
-from .build import lib_path
+from .build import lib_path, probes_path
 
 # op-tuple nibbles (include/fusedMM.h; reference fusedMM.h:18-73)
 VOP_NOOP, VOP_COPY_LHS, VOP_COPY_RHS, VOP_ADD, VOP_SUBL, VOP_SUBR, VOP_MAX, VOP_MIN, VOP_UDEF = \
@@ -26,19 +26,23 @@ MSG_SIGMOID = VOP_COPY_RHS | ROP_DOT | SOP_UDEF | VSC_MUL | AOP_ADD
 MSG_SPMM = VOP_COPY_RHS | ROP_NOOP | SOP_COPY | VSC_MUL | AOP_ADD
 MSG_GCN = VOP_COPY_RHS | ROP_NOOP | SOP_NOOP | VSC_NOOP | AOP_ADD
 
-SOP_KIND_HOST, SOP_KIND_IDENTITY, SOP_KIND_SIGMOID, SOP_KIND_TDIST, SOP_KIND_FR, SOP_KIND_LL, SOP_KIND_FA = \
-    -1, 0, 1, 2, 3, 4, 5
+SOP_KIND_HOST, SOP_KIND_IDENTITY, SOP_KIND_SIGMOID, SOP_KIND_TDIST, SOP_KIND_FR, SOP_KIND_LL, SOP_KIND_FA, \
+    SOP_KIND_TDIST_PLAIN = -1, 0, 1, 2, 3, 4, 5, 6
 
 SUCCESS, FAIL, VOP_FAIL, ROP_FAIL, AOP_FAIL, SOP_FAIL, VSC_FAIL = 0, 1, 2, 4, 8, 16, 32
 NOT_ENOUGH_MEM, UNDEFINED_USER_FUNCTION, NO_OPT_IMPL = -1, 64, 128
 
+# every symbol include/fusedMM.h and include/fusedmm_amd.h declare (sgfusedMM_csr / dgfusedMM_csr by precision)
 EXPORTS = ("fusedMM_csr", "fusedMM_csr_stream", "fusedMM_csr_stream_noalloc", "fusedMM_amd_init",
-           "fusedMM_amd_noalloc_capacity", "fusedMM_amd_index_bytes", "fusedMM_amd_value_bytes",
-           "fusedMM_amd_set_sop_kind", "fusedMM_amd_get_sop_kind", "fusedMM_amd_set_sop_callback",
-           "fusedMM_amd_set_opt", "fusedMM_amd_set_validate", "fusedMM_amd_set_split", "fusedMM_amd_timing",
-           "fusedMM_amd_timing_summary", "fusedMM_amd_timing_call", "fusedMM_amd_last_split", "fusedMM_amd_copy_probe",
-           "fusedMM_amd_read_probe", "fusedMM_amd_gather_probe", "fusedMM_amd_last_row_order", "fusedMM_amd_set_stage_callbacks", "fusedMM_amd_set_cache", "fusedMM_amd_invalidate", "fusedMM_amd_last_host_phases",
-           "fusedMM_amd_finalize")
+           "fusedMM_amd_init_noalloc", "fusedMM_amd_noalloc_capacity", "fusedMM_amd_index_bytes",
+           "fusedMM_amd_value_bytes", "fusedMM_amd_set_sop_kind", "fusedMM_amd_get_sop_kind",
+           "fusedMM_amd_set_sop_callback", "fusedMM_amd_set_stage_callbacks", "fusedMM_amd_set_opt",
+           "fusedMM_amd_set_validate", "fusedMM_amd_set_cache", "fusedMM_amd_invalidate",
+           "fusedMM_amd_last_host_phases", "fusedMM_amd_set_split", "fusedMM_amd_get_split", "fusedMM_amd_set_pack_rows", "fusedMM_amd_timing",
+           "fusedMM_amd_timing_summary", "fusedMM_amd_timing_call", "fusedMM_amd_last_split",
+           "fusedMM_amd_last_row_order", "fusedMM_amd_finalize")
+# the measuring aids of libfusedmm_amd_probes.so (csrc/fusedmm_probes.h): not part of the product's ABI
+PROBE_EXPORTS = ("fusedMM_amd_copy_probe", "fusedMM_amd_read_probe", "fusedMM_amd_gather_probe")
 
 _libs = {}
 
@@ -71,6 +75,7 @@ def load(index_bits=32, value_bits=32):
     lib.fusedMM_csr_stream_noalloc.argtypes = csr + [vp]
     lib.fusedMM_csr_stream_noalloc.restype = C.c_int
     lib.fusedMM_amd_init.restype = C.c_int
+    lib.fusedMM_amd_init_noalloc.restype = C.c_int
     lib.fusedMM_amd_noalloc_capacity.restype = C.c_int64
     gf = lib.sgfusedMM_csr if value_bits == 32 else lib.dgfusedMM_csr   # kernels.h:17-37 of the reference
     gf.argtypes = [C.c_char] + csr[1:]
@@ -93,12 +98,10 @@ def load(index_bits=32, value_bits=32):
     lib.fusedMM_amd_timing_call.restype = C.c_int
     lib.fusedMM_amd_last_split.argtypes = [C.POINTER(C.c_uint)] * 3
     lib.fusedMM_amd_last_split.restype = C.c_int
-    lib.fusedMM_amd_copy_probe.argtypes = [vp, vp, C.c_int64, vp]
-    lib.fusedMM_amd_copy_probe.restype = C.c_int
-    lib.fusedMM_amd_read_probe.argtypes = [vp, C.c_int64, C.c_int, C.c_int, C.c_int, vp, vp]
-    lib.fusedMM_amd_read_probe.restype = C.c_int
-    lib.fusedMM_amd_gather_probe.argtypes = [vp, C.c_int, vp, C.c_int64, C.c_int, C.c_int, C.c_int, vp, vp]
-    lib.fusedMM_amd_gather_probe.restype = C.c_int
+    lib.fusedMM_amd_get_split.argtypes = [C.POINTER(C.c_int64), C.POINTER(C.c_int)]
+    lib.fusedMM_amd_get_split.restype = None
+    lib.fusedMM_amd_set_pack_rows.argtypes = [C.c_int]
+    lib.fusedMM_amd_set_pack_rows.restype = C.c_int
     lib.fusedMM_amd_last_row_order.argtypes = [vp, vp, vp]
     lib.fusedMM_amd_last_row_order.restype = C.c_int
     lib.fusedMM_amd_set_stage_callbacks.argtypes = [vp, vp, vp, vp]
@@ -114,9 +117,32 @@ def load(index_bits=32, value_bits=32):
     return lib
 
 
+_probes = None
+
+
 def load_probes():
-    """The measuring aids (copy, read-stream and gather probes): bench.py's yardsticks, not part of the product ABI."""
-    return load(32, 32)
+    """dlopen libfusedmm_amd_probes.so, the measuring aids of the benchmark (copy, read-stream and
+    gather probes; csrc/fusedmm_probes.h): bench.py's yardsticks, not part of the product ABI."""
+    global _probes
+    if _probes is not None:
+        return _probes
+    try:
+        import torch  # noqa: F401  (one HIP runtime per process, as in load())
+    except ImportError:
+        pass
+    path = probes_path()
+    if not os.path.exists(path):
+        raise OSError("%s is not built; run `python -m fusedmm_amd.build`" % path)
+    lib = C.CDLL(path)
+    vp = C.c_void_p
+    lib.fusedMM_amd_copy_probe.argtypes = [vp, vp, C.c_int64, vp]
+    lib.fusedMM_amd_copy_probe.restype = C.c_int
+    lib.fusedMM_amd_read_probe.argtypes = [vp, C.c_int64, C.c_int, C.c_int, C.c_int, vp, vp]
+    lib.fusedMM_amd_read_probe.restype = C.c_int
+    lib.fusedMM_amd_gather_probe.argtypes = [vp, C.c_int, vp, C.c_int64, C.c_int, C.c_int, C.c_int, vp, vp]
+    lib.fusedMM_amd_gather_probe.restype = C.c_int
+    _probes = lib
+    return lib
 
 
 def _addr(a):

@@ -46,7 +46,7 @@ enum : int {
 enum : int { OP_GCN = 0, OP_SPMM = 1, OP_DOT = 2, OP_DIST = 3, OP_GENERIC = 4 };
 
 // Device-native bodies for SOP_UDEF (numbering shared with the public header).
-enum : int { SOP_IDENTITY = 0, SOP_SIGMOID = 1, SOP_TDIST = 2, SOP_FR = 3, SOP_LL = 4, SOP_FA = 5 };
+enum : int { SOP_IDENTITY = 0, SOP_SIGMOID = 1, SOP_TDIST = 2, SOP_FR = 3, SOP_LL = 4, SOP_FA = 5, SOP_TDIST_PLAIN = 6 };
 
 constexpr int kSigmoidTableSize = 2048;
 constexpr int kBlockThreads = 256;
@@ -125,6 +125,7 @@ struct Params {
    int kpad;
    int row_counters;       // claim counters in use: kRowCounters; 1 when the grid has fewer waves; 0: wave w takes chunk w
    int row_order;          // 0: decided from the classify kernel's sample; 1: first to last; 2: scattered stretches
+   int pack_rows;          // 1: groups of short rows are walked one row per sub-wave (sub-waves of 8 or 16 lanes)
 };
 
 // ---- wave primitives --------------------------------------------------------
@@ -308,6 +309,8 @@ __device__ __forceinline__ real_t sop_eval(int kind, real_t s, TabPtr tab)
       case SOP_FA:
          return (float)((double)sqrtf(s) + 1.0 / (double)s);
 #endif
+      case SOP_TDIST_PLAIN:
+         return (real_t)(1.0 / (1.0 + (double)s));   // the t-dist body without its constant -2 and its clamp
       default:
          return s;
    }
@@ -633,6 +636,7 @@ __device__ __forceinline__ void general_steps(Slice<R> &acc, const Slice<R> &xs,
          FMM_SOP_CASE(SOP_FR)
          FMM_SOP_CASE(SOP_LL)
          FMM_SOP_CASE(SOP_FA)
+         FMM_SOP_CASE(SOP_TDIST_PLAIN)
 #undef FMM_SOP_CASE
          default: break;
       }
@@ -877,6 +881,155 @@ __device__ __forceinline__ lds_table_t stage_table(const real_t *gtab, real_t *l
       __syncthreads();
    }
    return (lds_table_t)lds;      // read only when `need` held
+}
+
+// ---- short rows, one per sub-wave --------------------------------------------------
+// A wavefront walks a row with all its S = 64/L sub-waves: S*U edges are gathered at a
+// time.  Rows much shorter than that leave most of those gathers unused (a 16-edge row
+// at K=32 fills 16 of 64), and every row pays its own round of pointer, column-id and
+// store latency.  So a group of S consecutive rows (row ids g*S .. g*S+S-1, inside one
+// claim) whose longest row has  md <= S*U  edges and  ceil(md / U) <= (rows of the group
+// that have edges)  is walked with one row per sub-wave instead: the sub-wave gathers its
+// own row's edges U at a time, in edge order, into its own accumulator; nothing is merged
+// across sub-waves, and the S rows of X and Z are read and written as one contiguous
+// piece.  The rule compares the batches each way costs (ceil(md/U) against one per
+// non-empty row) and depends on the row pointers only, so the CPU oracle applies the same
+// rule; for such a row the sum runs over its edges in order in ONE accumulator (the
+// oracle's wavefront order with S = 1).
+template <int L, int U>
+__device__ __forceinline__ bool packs(int64_t md, int nz, int64_t heavy_deg)
+{
+   constexpr int S = 64 / L;
+   return nz > 0 && md <= (int64_t)(S * U) && md <= heavy_deg && (md + U - 1) / U <= (int64_t)nz;
+}
+
+// The group of S rows starting at `row_first` (wave-uniform), sub-wave s taking row
+// row_first + s with edge slots [jb, je) (per sub-wave; empty for rows past m), md the
+// longest row of the group.  All lanes of the wave call this together.
+template <int V, int L, int R, bool EXACT, int OP, int SOPK, int U, typename IdxT>
+__device__ __forceinline__ void packed_group(const Params<IdxT> &p, int64_t row_first, IdxT jb, IdxT je, int md, int lane,
+                                             lds_table_t tab)
+{
+   static_assert(L == 8 || L == 16, "sub-waves of 8 or 16 lanes");
+   constexpr int P = 16 / L;                 // column ids a lane holds per fetch: 16 ids per sub-wave and fetch
+   constexpr bool generic = (OP == OP_GENERIC);
+   constexpr bool uses_val = (OP == OP_SPMM || OP == OP_GENERIC);
+   const int sl = lane % L, base = lane - sl;
+   const int64_t row = row_first + lane / L;
+   const int deg = (int)(je - jb);           // <= S*U; 0 for empty rows and rows past m
+   const int sop_kind = SOPK >= 0 ? SOPK : p.sop_kind;
+   const bool reads_x = op_reads_x<OP>(p.imessage);
+   const int aop = p.imessage & 0xF0000;
+   real_t *zrow = p.z + row * p.ldz;
+
+   // ids [c0, c0 + 16) of the sub-wave's row: lane sl holds id c0 + sl (and c0 + 8 + sl when L == 8)
+   IdxT ids[P];
+   real_t vals[P];
+   auto fetch = [&](int c0, IdxT *id_out, real_t *val_out) {
+#pragma unroll
+      for (int q = 0; q < P; q++)
+      {
+         const int e = c0 + q * L + sl;
+         id_out[q] = 0;
+         val_out[q] = (real_t)0;
+         if (e < deg)
+         {
+            id_out[q] = p.indx[jb + (IdxT)e];
+            if (uses_val && p.val) val_out[q] = p.val[jb + (IdxT)e];
+         }
+      }
+   };
+   fetch(0, ids, vals);
+
+   Slice<R> xs, acc;
+   if (reads_x && deg > 0) load_slice<V, L, R, EXACT, true>(xs, p.x + row * p.ldx, sl, p.k);
+   else
+   {
+#pragma unroll
+      for (int r = 0; r < R; r++) xs.v[r] = zero4();
+   }
+   if (generic && deg > 0) load_slice<V, L, R, EXACT>(acc, zrow, sl, p.k);   // general rule: fold into the caller's Z
+   else
+   {
+#pragma unroll
+      for (int r = 0; r < R; r++) acc.v[r] = zero4();
+   }
+
+   for (int c0 = 0; c0 < md; c0 += 16)
+   {
+      IdxT nids[P];
+      real_t nvals[P];
+      if (c0 + 16 < md) fetch(c0 + 16, nids, nvals);     // wave-uniform: the next 16 ids while these are used
+      auto batch = [&](int b) {
+         if (c0 + b < md)                                 // wave-uniform
+         {
+         IdxT col[U];
+         real_t ev[U];
+         bool ok[U];
+         Slice<R> ys[U];
+#pragma unroll
+         for (int u = 0; u < U; u++)
+         {
+            const int i = b + u;                          // id i of the 16 fetched: register i / L, lane i % L
+            ok[u] = c0 + i < deg;
+            // (a select, not an indexed array: where the general pipeline keeps this loop rolled, b is not a constant)
+            const IdxT id_reg = (P == 1 || i < L) ? ids[0] : ids[P - 1];
+            const real_t val_reg = (P == 1 || i < L) ? vals[0] : vals[P - 1];
+            col[u] = chunk_entry<L>(id_reg, base + i % L);
+            ev[u] = uses_val ? chunk_entry<L>(val_reg, base + i % L) : (real_t)0;
+         }
+#pragma unroll
+         for (int u = 0; u < U; u++)
+         {
+            if (ok[u]) load_slice<V, L, R, EXACT>(ys[u], p.y + (int64_t)col[u] * p.ldy, sl, p.k);
+            else if (generic)
+            {
+#pragma unroll
+               for (int r = 0; r < R; r++) ys[u].v[r] = zero4();
+            }
+         }
+         if constexpr (generic)
+         {
+            const int left = md - (c0 + b);               // wave-uniform: the longest row's edges from here on
+            general_batch<L, R, U>(acc, xs, ys, ev, ok, left >= U ? U : left, sop_kind, p.imessage, tab);
+         }
+         else
+         {
+#pragma unroll
+            for (int u = 0; u < U; u++)
+               if (ok[u]) edge_step<L, R, OP>(acc, xs, ys[u], ev[u], sop_kind, tab);
+         }
+         }
+      };
+      if constexpr (generic)
+      {
+         for (int b = 0; b < 16; b += U) batch(b);        // the general pipeline's stages are large: kept as a loop
+      }
+      else
+      {
+#pragma unroll
+         for (int b = 0; b < 16; b += U) batch(b);
+      }
+      if (c0 + 16 < md)
+      {
+#pragma unroll
+         for (int q = 0; q < P; q++) { ids[q] = nids[q]; vals[q] = nvals[q]; }
+      }
+   }
+
+   if (deg > 0)
+   {
+      if (generic && aop == kAopNoop) return;             // no accumulate stage: Z is left alone
+      if (!generic && !p.beta_zero)
+      {
+         Slice<R> zin;
+         load_slice<V, L, R, EXACT>(zin, zrow, sl, p.k);
+         map2(acc, zin, acc, [](real_t a, real_t b) { return a + b; });
+      }
+      store_slice<V, L, R, EXACT, true>(zrow, acc, sl, p.k);
+   }
+   else if (!generic && p.beta_zero && row < p.m)
+      store_slice<V, L, R, EXACT, true>(zrow, acc, sl, p.k);   // empty row under the overwrite rule: zeros
 }
 
 // Does the row phase take the stretches of 64 chunks in scattered order?  When rows are claimed dynamically,
@@ -1265,12 +1418,41 @@ __device__ __forceinline__ void rows_phase(const Params<IdxT> &p, lds_table_t ta
    if (nc > 0 && lane == 0) claimed = atomicAdd(&p.ctr->rows[cur].next, 1ull);
    // rows of this claim that have edges, one bit per row: while a row is walked, the
    // first column ids and the X slice of the next such row are already on their way
-   const unsigned int has_edges = (unsigned int)__ballot(lane < kRowsPerClaim && my_e > my_b);
+   unsigned int has_edges = (unsigned int)__ballot(lane < kRowsPerClaim && my_e > my_b);
+   unsigned int packed_rows = 0u;   // rows of this claim that were walked one per sub-wave
+   if constexpr (V == 4 && L <= 16)
+   {
+      if (p.pack_rows && !(generic && aop == kAopNoop))
+      {
+         constexpr int S = 64 / L;
+         for (int g0 = 0; g0 < kRowsPerClaim; g0 += S)
+         {
+            const unsigned int gmask = ((1u << S) - 1u) << g0;
+            const int nz = __builtin_popcount(has_edges & gmask);
+            int64_t md = 0;
+#pragma unroll
+            for (int t = g0; t < g0 + S; t++)
+            {
+               const int64_t d = (int64_t)lane_value<IdxT>(my_e, t) - (int64_t)lane_value<IdxT>(my_b, t);
+               md = d > md ? d : md;
+            }
+            if (packs<L, U>(md, nz, p.heavy_deg))
+            {
+               // sub-wave s takes row row0 + g0 + s: its pointers are in lane g0 + s
+               const IdxT gb = chunk_entry<L>(my_b, g0 + lane / L), ge = chunk_entry<L>(my_e, g0 + lane / L);
+               packed_group<V, L, R, EXACT, OP, SOPK, U, IdxT>(p, row0 + g0, gb, ge > gb ? ge : gb, (int)md, lane, tab);
+               packed_rows |= gmask;
+            }
+         }
+         has_edges &= ~packed_rows;
+      }
+   }
    EdgeChunk<IdxT> first;
    Slice<R> xs_next;
    int fetched_t = -1;        // row of this claim whose first chunk `first` (and X slice `xs_next`) hold
    for (int t = 0; t < kRowsPerClaim && row0 + t < p.m; t++)
    {
+      if ((packed_rows >> t) & 1u) continue;
       const int64_t row = row0 + t;
       const IdxT jb = lane_value<IdxT>(my_b, t);
       const IdxT je = lane_value<IdxT>(my_e, t);
@@ -1506,282 +1688,6 @@ __global__ __launch_bounds__(kBlockThreads) void merge_kernel(const Params<IdxT>
          }
       }
    }
-}
-
-// ---- host-callback SOP, pass 1: s[j] = ROP(X[i], VOP(X[i], Y[c])) for every edge slot ----
-// One wave per row (static stride; this path exists for compatibility, the
-// host evaluates the caller's SOP_UDEF_FUNC on s[] before the accumulate pass).
-template <int V, int L, int R, bool EXACT, int U, typename IdxT>
-__global__ __launch_bounds__(kBlockThreads) void edge_scalar_kernel(const Params<IdxT> p, real_t *s_out, int accumulate)
-{
-   constexpr int S = 64 / L;
-   const int lane = threadIdx.x & 63;
-   const int sub = lane / L, sl = lane % L;
-   const int64_t wave0 = (int64_t)blockIdx.x * kWavesPerBlock + (threadIdx.x >> 6);
-   const int64_t nwaves = (int64_t)gridDim.x * kWavesPerBlock;
-   const int vop = p.imessage & 0xF, rop = p.imessage & 0xF0;
-   for (int64_t row = wave0; row < p.m; row += nwaves)
-   {
-      const IdxT jb = wave_uniform<IdxT>(p.pntrb[row]);
-      const IdxT je = wave_uniform<IdxT>(p.pntre[row]);
-      Slice<R> xs;
-      load_slice<V, L, R, EXACT>(xs, p.x + row * p.ldx, sl, p.k);
-      // slot numbers in 64 bits: an int32 slot next to 2^31 must not wrap when stepped past je
-      const int64_t je64 = (int64_t)je;
-      for (int64_t j0 = (int64_t)jb; j0 < je64; j0 += S * U)
-      {
-#pragma unroll
-         for (int u = 0; u < U; u++)
-         {
-            const int64_t j = j0 + sub + u * S;
-            if (j < je64)
-            {
-               Slice<R> ys, t;
-               load_slice<V, L, R, EXACT>(ys, p.y + (int64_t)p.indx[j] * p.ldy, sl, p.k);
-               const real_t scal = vop_rop<L, R>(t, xs, ys, p.val ? p.val[j] : (real_t)0, vop, rop);
-               // every ROP is a sum over elements, so column slabs of a wide row add up
-               if (sl == 0) s_out[j] = accumulate ? s_out[j] + scal : scal;
-            }
-         }
-      }
-   }
-}
-
-// d[j] = SOP(s[j]) in place, for the wide-row path where the ROP result is
-// assembled from column slabs before the scalar op can be applied.
-__global__ __launch_bounds__(kBlockThreads) void apply_sop_kernel(real_t *s, int64_t n, int sop_kind, const real_t *tab)
-{
-   for (int64_t i = (int64_t)blockIdx.x * kBlockThreads + threadIdx.x; i < n; i += (int64_t)gridDim.x * kBlockThreads)
-      s[i] = sop_eval(sop_kind, s[i], tab);
-}
-
-// ---- the pipeline stage by stage over materialised edges ---------------------------
-// For tuples in which VOP, ROP, VSC or AOP is the caller's host function: the
-// per-edge vector T[j][0..k) and scalar s[j] live in device buffers indexed by edge
-// slot, so that a host pass can stand in for any stage while the library's own
-// stages stay on the GPU.  One wavefront per row.  Every built-in stage evaluates in
-// the reference's own order (fusedMM.c:28-333: element by element, sums left to
-// right, separate multiply and add), so the results are the reference's bits.
-
-// T[j] = VOP(X[i], Y[indx[j]])
-template <typename IdxT>
-__global__ __launch_bounds__(kBlockThreads) void stage_vop_kernel(const Params<IdxT> p, real_t *T)
-{
-   const int lane = threadIdx.x & 63;
-   const int vop = p.imessage & 0xF;
-   const int64_t wave0 = (int64_t)blockIdx.x * kWavesPerBlock + (threadIdx.x >> 6);
-   for (int64_t i = wave0; i < p.m; i += (int64_t)gridDim.x * kWavesPerBlock)
-   {
-      const real_t *xr = p.x + i * p.ldx;
-      for (int64_t j = (int64_t)p.pntrb[i]; j < (int64_t)p.pntre[i]; j++)
-      {
-         const real_t *yr = p.y + (int64_t)p.indx[j] * p.ldy;
-         real_t *t = T + j * p.k;
-         for (int e = lane; e < p.k; e += 64)
-         {
-            const real_t a = xr[e], b = yr[e];
-            real_t v;
-            switch (vop)
-            {
-               case kVopCopyLhs: v = a; break;
-               case kVopCopyRhs: v = b; break;
-               case kVopAdd: v = a + b; break;
-               case kVopSubl: v = -a + b; break;
-               case kVopSubr: v = a - b; break;
-               case kVopMax: v = a > b ? a : b; break;
-               default: v = a < b ? a : b; break;
-            }
-            t[e] = v;
-         }
-      }
-   }
-}
-
-// s[j] = ROP(X[i], T[j]); a lane owns an edge and sums its k terms left to right.
-// (ROP_NOOP is not launched: s[j] stays the edge value.)
-template <typename IdxT>
-__global__ __launch_bounds__(kBlockThreads) void stage_rop_kernel(const Params<IdxT> p, const real_t *T, real_t *s)
-{
-   const int lane = threadIdx.x & 63;
-   const int rop = p.imessage & 0xF0;
-   const int64_t wave0 = (int64_t)blockIdx.x * kWavesPerBlock + (threadIdx.x >> 6);
-   for (int64_t i = wave0; i < p.m; i += (int64_t)gridDim.x * kWavesPerBlock)
-   {
-      const real_t *xr = p.x + i * p.ldx;
-      for (int64_t j = (int64_t)p.pntrb[i] + lane; j < (int64_t)p.pntre[i]; j += 64)
-      {
-         const real_t *t = T + j * p.k;
-         real_t acc = (real_t)0;
-         for (int e = 0; e < p.k; e++)
-         {
-            real_t term;
-            switch (rop)
-            {
-               case kRopDot: term = xr[e] * t[e]; break;
-               case kRopAddLhs: term = xr[e]; break;
-               case kRopAddRhs: term = t[e]; break;
-               case kRopNormL: term = xr[e] * xr[e]; break;
-               default: term = t[e] * t[e]; break;   // kRopNormR
-            }
-            acc = acc + term;
-         }
-         s[j] = acc;
-      }
-   }
-}
-
-// T[j] = VSC(s[j], T[j]) for the edge slots of the processed rows
-template <typename IdxT>
-__global__ __launch_bounds__(kBlockThreads) void stage_vsc_kernel(const Params<IdxT> p, real_t *T, const real_t *s)
-{
-   const int lane = threadIdx.x & 63;
-   const int vsc = p.imessage & 0xF000;
-   const int64_t wave0 = (int64_t)blockIdx.x * kWavesPerBlock + (threadIdx.x >> 6);
-   for (int64_t i = wave0; i < p.m; i += (int64_t)gridDim.x * kWavesPerBlock)
-      for (int64_t j = (int64_t)p.pntrb[i]; j < (int64_t)p.pntre[i]; j++)
-      {
-         const real_t d = s[j];
-         real_t *t = T + j * p.k;
-         for (int e = lane; e < p.k; e += 64) t[e] = (vsc == kVscMul) ? d * t[e] : d + t[e];
-      }
-}
-
-// Z[i] = AOP(Z[i], T[j]) over the row's edges in order; a lane owns a column.
-template <typename IdxT>
-__global__ __launch_bounds__(kBlockThreads) void stage_aop_kernel(const Params<IdxT> p, const real_t *T)
-{
-   const int lane = threadIdx.x & 63;
-   const int aop = p.imessage & 0xF0000;
-   const int64_t wave0 = (int64_t)blockIdx.x * kWavesPerBlock + (threadIdx.x >> 6);
-   for (int64_t i = wave0; i < p.m; i += (int64_t)gridDim.x * kWavesPerBlock)
-   {
-      const int64_t jb = (int64_t)p.pntrb[i], je = (int64_t)p.pntre[i];
-      if (je <= jb) continue;
-      real_t *zr = p.z + i * p.ldz;
-      for (int e = lane; e < p.k; e += 64)
-      {
-         real_t z = zr[e];
-         for (int64_t j = jb; j < je; j++)
-         {
-            const real_t t = T[j * p.k + e];
-            if (aop == kAopAdd) z = z + t;
-            else if (aop == kAopMax) z = z > t ? z : t;
-            else z = z < t ? z : t;
-         }
-         zr[e] = z;
-      }
-   }
-}
-
-// Optional operand check (off by default, like the reference, which trusts its
-// caller): a column id outside [0, n) or a row with pntre < pntrb would make the
-// kernels read outside Y.  Sets flag[0] when anything is wrong.
-template <typename IdxT>
-__global__ __launch_bounds__(kBlockThreads) void validate_kernel(const Params<IdxT> p, int64_t n, unsigned int *flag)
-{
-   const int lane = threadIdx.x & 63;
-   const int64_t wave0 = (int64_t)blockIdx.x * kWavesPerBlock + (threadIdx.x >> 6);
-   const int64_t nwaves = (int64_t)gridDim.x * kWavesPerBlock;
-   bool bad = false;
-   for (int64_t row = wave0; row < p.m; row += nwaves)
-   {
-      const IdxT jb = p.pntrb[row], je = p.pntre[row];
-      if (je < jb || jb < 0) { bad = true; continue; }
-      for (int64_t j = (int64_t)jb + lane; j < (int64_t)je; j += 64)   // 64-bit: no wrap next to 2^31
-      {
-         const IdxT c = p.indx[j];
-         if (c < 0 || (int64_t)c >= n) bad = true;
-      }
-   }
-   if (bad) atomicOr(flag, 1u);
-}
-
-// Z[i, 0:k] = 0 for i < m (the overwrite rule of the pattern tuples, when the
-// accumulate pass that follows can only add).
-__global__ __launch_bounds__(kBlockThreads) void zero_rows_kernel(real_t *z, int64_t m, int64_t k, int64_t ldz)
-{
-   const int64_t total = m * k;
-   for (int64_t i = (int64_t)blockIdx.x * kBlockThreads + threadIdx.x; i < total; i += (int64_t)gridDim.x * kBlockThreads)
-      z[(i / k) * ldz + (i % k)] = (real_t)0;
-}
-
-// Plain 16-byte copy of known size: the yardstick the HBM traffic counters
-// (FETCH_SIZE / WRITE_SIZE) of the kernels above are scaled by.
-__global__ __launch_bounds__(kBlockThreads) void copy_probe_kernel(float4 *dst, const float4 *src, int64_t n16)
-{
-   for (int64_t i = (int64_t)blockIdx.x * kBlockThreads + threadIdx.x; i < n16; i += (int64_t)gridDim.x * kBlockThreads)
-      dst[i] = src[i];
-}
-
-
-// Read-only stream of known size: every thread keeps U independent 16-byte loads
-// in flight and folds what it read into one word, stored only if it is a value
-// the data never produces, so the loads cannot be dropped and nothing is
-// written.  The yardstick for what this GPU's HBM delivers to reads alone.
-typedef unsigned int probe16_t __attribute__((ext_vector_type(4)));
-template <int U, bool NT>
-__global__ __launch_bounds__(kBlockThreads) void read_probe_kernel(const probe16_t *src, int64_t n16, unsigned int *sink)
-{
-   const int64_t stride = (int64_t)gridDim.x * kBlockThreads;
-   unsigned int acc = 0u;
-   int64_t i = (int64_t)blockIdx.x * kBlockThreads + threadIdx.x;
-   for (; i + (U - 1) * stride < n16; i += U * stride)
-   {
-      probe16_t v[U];
-#pragma unroll
-      for (int u = 0; u < U; u++)
-         v[u] = NT ? __builtin_nontemporal_load(src + i + u * stride) : src[i + u * stride];
-#pragma unroll
-      for (int u = 0; u < U; u++) acc ^= v[u].x ^ v[u].y ^ v[u].z ^ v[u].w;
-   }
-   for (; i < n16; i += stride)
-   {
-      const probe16_t v = src[i];
-      acc ^= v.x ^ v.y ^ v.z ^ v.w;
-   }
-   if (acc == 0x9E3779B9u) *sink = acc;
-}
-
-// Read-only gather of whole rows: row ids[j] of `row16` 16-byte pieces each (a power of
-// two up to 64 * R), for j < n_ids, in the order given; a wavefront takes 64 / L rows at
-// a time on L = min(64, row16) lanes each and keeps U such steps in flight.  Nothing but
-// the loads and an exclusive-or: the yardstick for what the memory system delivers to
-// gathers of rows of this size, as read_probe_kernel is for a stream.
-template <int U, int R, bool NT>
-__global__ __launch_bounds__(kBlockThreads) void gather_probe_kernel(const probe16_t *src, int row16, const unsigned int *ids,
-                                                                     int64_t n_ids, unsigned int *sink)
-{
-   const int lane = threadIdx.x & 63;
-   const int L = row16 / R, S = 64 / L;
-   const int sub = lane / L, sl = lane % L;
-   const int64_t wave = ((int64_t)blockIdx.x * kBlockThreads + threadIdx.x) >> 6;
-   const int64_t nwaves = (int64_t)gridDim.x * (kBlockThreads / 64);
-   unsigned int acc = 0u;
-   for (int64_t b = wave * S * U; b < n_ids; b += nwaves * S * U)
-   {
-      int64_t row[U];
-#pragma unroll
-      for (int u = 0; u < U; u++)
-      {
-         const int64_t j = b + u * S + sub;
-         row[u] = j < n_ids ? (int64_t)ids[j] : -1;
-      }
-      probe16_t v[U][R];
-#pragma unroll
-      for (int u = 0; u < U; u++)
-#pragma unroll
-         for (int r = 0; r < R; r++)
-         {
-            const probe16_t *at = src + row[u] * row16 + r * L + sl;
-            if (row[u] >= 0) v[u][r] = NT ? __builtin_nontemporal_load(at) : *at;
-            else v[u][r] = probe16_t{0u, 0u, 0u, 0u};
-         }
-#pragma unroll
-      for (int u = 0; u < U; u++)
-#pragma unroll
-         for (int r = 0; r < R; r++) acc ^= v[u][r].x ^ v[u][r].y ^ v[u][r].z ^ v[u][r].w;
-   }
-   if (acc == 0x9E3779B9u) *sink = acc;
 }
 
 }  // namespace fmm

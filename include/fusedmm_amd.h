@@ -24,6 +24,11 @@ extern "C" {
 #define FUSEDMM_SOP_KIND_FR         3  /* d = 1 + 1/s                    (:635-639) */
 #define FUSEDMM_SOP_KIND_LL         4  /* d = log2(1 + sqrt(s))          (:649-653) */
 #define FUSEDMM_SOP_KIND_FA         5  /* d = sqrt(s) + 1/s              (:656-660) */
+/* The t-distribution weight as it is usually written, d = 1/(1+s): the tester's body (kind 2) is this times
+ * the constant -2, clamped to [-5, 5], which never binds for s >= 0.  No body of the tester computes it; a
+ * caller who wants it from the reference writes it as a SOP_UDEF_FUNC, and this kind gives the bits such a
+ * function written with the tester's conventions gives: (VALUETYPE)(1.0 / (1.0 + s)), formed in double. */
+#define FUSEDMM_SOP_KIND_TDIST_PLAIN 6
 
 /*
  * Choose what SOP_UDEF means for later fusedMM_csr calls of this process.
@@ -31,7 +36,9 @@ extern "C" {
  * (kernels/CONFIG/make.base:339-345 builds one executable per -D<KIND>_UDEF).
  * Returns the previous kind, or -2 for an unknown kind.  The initial kind comes
  * from the environment variable FUSEDMM_SOP_KIND (host, identity, sigmoid,
- * tdist, fr, ll, fa) and is "host" when that is unset.
+ * tdist, fr, ll, fa, tdist_plain) and is "host" when that is unset.  A call of this function
+ * overrides the variable, whenever it is made (the same holds for every setter below whose
+ * setting also has a variable).
  */
 int fusedMM_amd_set_sop_kind(int kind);
 int fusedMM_amd_get_sop_kind(void);
@@ -137,6 +144,13 @@ int64_t fusedMM_amd_noalloc_capacity(void);
  * while it is switched on.  Returns a fusedMM status code. */
 int fusedMM_amd_init(void);
 
+/* The part of fusedMM_amd_init() that fusedMM_csr_stream_noalloc needs, for callers that must not
+ * allocate device memory at set-up either: looks up the static array's address on the current
+ * device, copies the sigmoid table there and clears its counters (blocking copies: not inside a
+ * capture).  No hipMalloc; the ordinary entry points still make their small allocations on their
+ * own first use.  No counterpart in the reference.  Returns a fusedMM status code. */
+int fusedMM_amd_init_noalloc(void);
+
 /*
  * The reference's second-level entry (kernels/include/kernels.h:32-37,
  * kernels/src/kernels.c:456-631): tkern 'g' gcn, 'm' spmm, 's' sigmoid,
@@ -206,6 +220,18 @@ int fusedMM_amd_last_host_phases(double *upload_ms, double *kernels_ms, double *
  * are cut into segments of `seg_len` edges (0, 0 restores the K-dependent
  * defaults).  For tests and experiments. */
 void fusedMM_amd_set_split(int64_t heavy_deg, int seg_len);
+/* The values in force (0: the K-dependent default): what fusedMM_amd_set_split() last set, or else what
+ * the environment variable FUSEDMM_SPLIT=heavy_deg,seg_len gave. */
+void fusedMM_amd_get_split(int64_t *heavy_deg, int *seg_len);
+
+/* Short rows one per group of lanes.  For K <= 64 a wavefront holds 4 (K > 32) or 8 neighbour rows at a
+ * time; a group of that many consecutive CSR rows whose longest has no more than 8 edges per non-empty row
+ * of the group (and at most 32 / 64 edges) is processed with one row per group of lanes, every row's edges
+ * in order, instead of one row after the other across the whole wavefront.  1 (default; also
+ * FUSEDMM_PACK_ROWS=on|auto) enables it, 0 (FUSEDMM_PACK_ROWS=off) disables it.  Which rows are taken that
+ * way depends on the row pointers only; it changes the order in which such a row's edges are summed (same
+ * values to rounding) and nothing else.  Returns the previous setting. */
+int fusedMM_amd_set_pack_rows(int enable);
 
 /*
  * Per-kernel timing with HIP events on the stream the kernels run on.
@@ -235,32 +261,6 @@ int fusedMM_amd_last_split(unsigned int *heavy_rows, unsigned int *segments, uns
  * Results do not depend on it.  The environment variable FUSEDMM_ROW_ORDER=plain | scattered | auto
  * (read once, at the first call) overrides the choice.  Waits for the GPU. */
 int fusedMM_amd_last_row_order(int *scattered, unsigned int *edges_lower_half, unsigned int *edges_upper_half);
-
-/* Copy `bytes` (a multiple of 16, device memory, 16-byte aligned) with a plain
- * grid-stride kernel on `stream`, asynchronously.  A measuring aid: hardware
- * traffic counters of the kernels are scaled by what they read for this copy
- * of known size. */
-int fusedMM_amd_copy_probe(void *dst, const void *src, int64_t bytes, void *stream);
-
-/* Read `bytes` (a multiple of 16, device memory, 16-byte aligned) with a grid of
- * blocks_per_cu workgroups per compute unit, each thread keeping `in_flight`
- * (2, 4, 8 or 16) independent 16-byte loads outstanding, non-temporal or not;
- * nothing is written (`sink`, 4 bytes of device memory, only keeps the loads
- * alive).  A measuring aid: what this GPU's HBM delivers to reads alone, next to
- * which the gather kernels' bandwidth is quoted. */
-int fusedMM_amd_read_probe(const void *src, int64_t bytes, int blocks_per_cu, int in_flight, int nontemporal,
-                           void *sink, void *stream);
-
-/* Gather `n_ids` whole rows of `row_bytes` bytes (a power of two, 16..2048) from
- * `src` at the row numbers ids[0..n_ids) (device memory; the caller keeps them
- * inside `src`), in that order, with blocks_per_cu workgroups per compute unit
- * and `in_flight` (4, 8 or 16; 4 or 8 for 2048-byte rows) rows outstanding per
- * group of lanes that shares a row; nothing else is computed and nothing is
- * written.  A measuring aid: what the memory system delivers to gathers of rows
- * of the size a benchmark gathers, where fusedMM_amd_read_probe gives the rate of
- * a plain stream. */
-int fusedMM_amd_gather_probe(const void *src, int row_bytes, const unsigned int *ids, int64_t n_ids, int blocks_per_cu,
-                             int in_flight, int nontemporal, void *sink, void *stream);
 
 /* Release every device buffer the library holds (work queues, staging). */
 void fusedMM_amd_finalize(void);

@@ -17,6 +17,11 @@
  *          SOP_UDEF_FUNC bodies through oracle/_ref (tests/test_oracle_ref.py),
  *          committed as tests/golden/sop_*.npz; closed forms sigma(0)=0.5,
  *          saturation beyond +-5, monotonicity.
+ *        ORC_SOP_TDIST_PLAIN (1/(1+val); no such body in the harness) - closed
+ *          form in exact arithmetic on dyadic arguments; -2 * plain == the TDIST
+ *          body bit for bit wherever its clamp does not bind (a power-of-two
+ *          factor commutes with the one rounding); dense fp64 brute force of the
+ *          whole op; X == Y rows contribute exactly zero.
  *   orc_fusedmm_generic_*  - bit-compared with the reference's generic
  *          fusedMM_csr (compiled from /root/reference/fusedMM.c) on seeded
  *          inputs; scipy CSR @ Y for the spmm/gcn tuples; dense brute force.
@@ -74,7 +79,12 @@ enum {
    ORC_SOP_TDIST = 2,    /* clamp(-2/(1+val), +-5)          (:642-646)  */
    ORC_SOP_FR = 3,       /* 1 + 1/val                       (:635-639)  */
    ORC_SOP_LL = 4,       /* log2(1 + sqrt(val))             (:649-653)  */
-   ORC_SOP_FA = 5        /* sqrt(val) + 1/val               (:656-660)  */
+   ORC_SOP_FA = 5,       /* sqrt(val) + 1/val               (:656-660)  */
+   /* Not a body of the harness: the t-distribution weight as usually written,
+    * 1/(1+val), i.e. the TDIST body without its constant -2 and its clamp, in the
+    * harness's conventions (double literals, one rounding).  Pinned by its closed
+    * form and by its exact relation to ORC_SOP_TDIST (tests/test_oracle_pins.py). */
+   ORC_SOP_TDIST_PLAIN = 6
 };
 
 /* ---- value-type dependent part, compiled for float and double ---- */

@@ -25,6 +25,28 @@ def layout_for(k, vec_ok=True):
 
 
 MAX_SEGS_PER_ROW = 512   # kMaxSegsPerRow of the kernels: longer rows get longer segments
+ROWS_PER_CLAIM = 8       # kRowsPerClaim
+
+
+def packed_rows(g, m, k, vbits, heavy_deg, vec_ok=True, pack=True):
+    """Which of the first m rows the library walks one per sub-wave (packed_group of the kernels): for sub-waves
+    of 8 or 16 lanes (K <= 64, 16-byte layout), a group of S = 64/L consecutive rows, groups aligned at multiples
+    of S, whose longest row has md <= S*U edges (and is not split) and ceil(md / U) <= (non-empty rows of the
+    group).  U is the number of gathers a sub-wave keeps in flight: 8, or 4 in double precision.  Such a row is
+    summed over its edges in order in one accumulator."""
+    V, L, S = layout_for(k, vec_ok)
+    out = np.zeros(m, bool)
+    if not pack or V != 4 or L > 16 or m == 0:
+        return out
+    U = 8 if vbits == 32 else 4
+    deg = (g["pntre"][:m].astype(np.int64) - g["pntrb"][:m].astype(np.int64))
+    deg = np.maximum(deg, 0)
+    pad = (-m) % S
+    d2 = np.concatenate([deg, np.zeros(pad, np.int64)]).reshape(-1, S)
+    md = d2.max(1)
+    nz = (d2 > 0).sum(1)
+    ok = (nz > 0) & (md <= S * U) & (md <= heavy_deg) & (-(-md // U) <= nz)
+    return np.repeat(ok, S)[:m]
 
 
 def default_split(k, vbits=32):
@@ -76,9 +98,10 @@ def last_split(bits=32, vbits=32):
     return h.value, s.value, o.value
 
 
-def oracle_mirror(oracle, tkern, g, X, Y, Z0, beta, sop_kind, k, heavy_deg, seg_len, vec_ok=True, m=None):
+def oracle_mirror(oracle, tkern, g, X, Y, Z0, beta, sop_kind, k, heavy_deg, seg_len, vec_ok=True, m=None, pack=True, packed=None):
     """What the library computes, operation for operation: rows up to heavy_deg
-    edges in wavefront order; longer rows cut into seg_len-edge segments (at
+    edges in wavefront order (short rows that the library walks one per sub-wave, packed_rows(), with a
+    single accumulator); longer rows cut into seg_len-edge segments (at
     most MAX_SEGS_PER_ROW per row), each reduced in wavefront order; the merge
     block's G thread groups fold segments g, g+G, ... in ascending order from
     zero, the group sums are added in ascending g, then Z is added when beta != 0."""
@@ -86,7 +109,22 @@ def oracle_mirror(oracle, tkern, g, X, Y, Z0, beta, sop_kind, k, heavy_deg, seg_
     V, L, S = layout_for(k, vec_ok)
     ot = "t" if tkern == "f" else tkern
     Z = Z0.copy()
-    oracle.opt(ot, g, X, Y, Z, beta=beta, sop_kind=sop_kind, mode=2, V=V, L=L, S=S, m=m)
+    vbits = 32 if Z0.dtype == np.float32 else 64
+    if packed is None:      # (a caller checking a window of rows passes the window's part of the whole matrix's mask)
+        packed = packed_rows(g, m, k, vbits, heavy_deg, vec_ok, pack)
+    if packed.all() and m > 0:
+        oracle.opt(ot, g, X, Y, Z, beta=beta, sop_kind=sop_kind, mode=2, V=V, L=L, S=1, m=m, k=k)
+    else:
+        oracle.opt(ot, g, X, Y, Z, beta=beta, sop_kind=sop_kind, mode=2, V=V, L=L, S=S, m=m, k=k)
+        if packed.any():
+            # the rows walked one per sub-wave, as a sub-problem of their own: same operands, one accumulator per row
+            rows = np.nonzero(packed)[0]
+            gp = dict(g)
+            gp.update(rows=rows.size, pntrb=np.ascontiguousarray(g["pntrb"][rows]), pntre=np.ascontiguousarray(g["pntre"][rows]))
+            Xp = None if X is None else np.ascontiguousarray(X[rows])
+            Zp = np.ascontiguousarray(Z0[rows])
+            oracle.opt(ot, gp, Xp, Y, Zp, beta=beta, sop_kind=sop_kind, mode=2, V=V, L=L, S=1, k=k)
+            Z[rows] = Zp
     deg = (g["pntre"][:m].astype(np.int64) - g["pntrb"][:m].astype(np.int64))
     heavy = np.nonzero(deg > heavy_deg)[0]
     if heavy.size == 0:
@@ -105,7 +143,7 @@ def oracle_mirror(oracle, tkern, g, X, Y, Z0, beta, sop_kind, k, heavy_deg, seg_
     X2 = None if X is None else np.ascontiguousarray(X[np.array(owner)])
     np_v = Z0.dtype.type
     P = np.zeros((len(pb), k), np_v)
-    oracle.opt(ot, g2, X2, Y, P, beta=0.0, sop_kind=sop_kind, mode=2, V=V, L=L, S=S)
+    oracle.opt(ot, g2, X2, Y, P, beta=0.0, sop_kind=sop_kind, mode=2, V=V, L=L, S=S, k=k)
     owner = np.array(owner)
     G = max(1, 256 // min(k, 256))          # merge kernel: groups of a 256-thread block
     for r in heavy:
@@ -116,7 +154,7 @@ def oracle_mirror(oracle, tkern, g, X, Y, Z0, beta, sop_kind, k, heavy_deg, seg_
             for q in mine[grp::G]:
                 a = (a + P[q]).astype(np_v)
             total = a if total is None else (total + a).astype(np_v)
-        Z[r] = total if beta == 0.0 else (Z0[r] + total).astype(np_v)
+        Z[r, :k] = total if beta == 0.0 else (Z0[r, :k] + total).astype(np_v)
     return Z
 
 

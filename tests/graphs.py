@@ -150,3 +150,29 @@ def udef_stage_tuples():
             msgs.append(stages[0] | stages[1] | stages[2] | stages[3] | stages[4])
     msgs.append(0xF | 0xF0 | 0xF00 | 0xF000 | 0x00000)   # no accumulate stage: Z untouched
     return np.array(sorted(set(msgs)), np.int32)
+
+
+def boundary_graph(bits=32, cols=500, seed=21):
+    """For the rule that walks short rows one per sub-wave (gpu_api.packed_rows).  Groups of 8 (and of 4) consecutive rows built around every edge of the rule: all rows at the longest
+    length that still packs, one row one edge too long, a single long row among empty ones, all empty, all
+    one edge, lengths 1..8 and 57..64, a group that straddles the end of the matrix (the row count is not a
+    multiple of 8), and Poisson-like lengths in between."""
+    rng = np.random.Generator(np.random.Philox(key=[seed, 0]))
+    groups = [
+        [64] * 8, [65] + [64] * 7, [64, 0, 0, 0, 0, 0, 0, 0], [8, 0, 0, 0, 0, 0, 0, 0], [9, 0, 0, 0, 0, 0, 0, 0],
+        [16, 16, 0, 0, 0, 0, 0, 0], [17, 16, 0, 0, 0, 0, 0, 0], [0] * 8, [1] * 8, [1, 2, 3, 4, 5, 6, 7, 8],
+        [57, 58, 59, 60, 61, 62, 63, 64], [32, 32, 32, 32, 0, 0, 0, 0], [33, 32, 32, 32, 1, 1, 1, 1],
+        [32, 1, 1, 1, 32, 0, 0, 0], [24, 24, 24, 0, 24, 24, 0, 0], [40, 3, 0, 0, 0, 12, 12, 12],
+    ]
+    for _ in range(30):
+        groups.append(list(rng.poisson(16, 8)))
+    for _ in range(10):
+        groups.append(list(rng.poisson(4, 8)))
+    groups.append([5, 9, 13])              # the last claim is short: rows past m must stay untouched
+    deg = np.array([d for grp in groups for d in grp], np.int64)
+    rowptr = np.zeros(deg.size + 1, np.int64)
+    np.cumsum(deg, out=rowptr[1:])
+    indx = rng.integers(0, cols, int(rowptr[-1]), dtype=np.int64)
+    g = synth.graph_from_rowptr(deg.size, cols, rowptr, indx, None, bits)
+    g["val"] = synth.edge_values(g["nnz"], seed)
+    return g

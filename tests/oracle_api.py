@@ -12,8 +12,8 @@ import numpy as np
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 ORACLE_DIR = os.path.join(ROOT, "oracle")
 
-SOP_IDENTITY, SOP_SIGMOID, SOP_TDIST, SOP_FR, SOP_LL, SOP_FA = range(6)
-SOP_NAMES = {"identity": 0, "sigmoid": 1, "tdist": 2, "fr": 3, "ll": 4, "fa": 5}
+SOP_IDENTITY, SOP_SIGMOID, SOP_TDIST, SOP_FR, SOP_LL, SOP_FA, SOP_TDIST_PLAIN = range(7)
+SOP_NAMES = {"identity": 0, "sigmoid": 1, "tdist": 2, "fr": 3, "ll": 4, "fa": 5, "tdist_plain": 6}
 
 # op tuples the reference harness sends (test/fusedMMtime.cpp:731-753)
 MSG = {
@@ -52,12 +52,30 @@ def _load(name):
     return C.CDLL(path)
 
 
+def host_has_avx512():
+    """Does this host's CPU offer what -march=x86-64-v4 code needs?"""
+    try:
+        for line in open("/proc/cpuinfo"):
+            if line.startswith("flags"):
+                have = set(line.split(":", 1)[1].split())
+                return {"avx512f", "avx512bw", "avx512cd", "avx512dq", "avx512vl"} <= have
+    except OSError:
+        pass
+    return False
+
+
 class Oracle:
-    """The CPU restatement.  fast=True loads the -O3 build (baseline timing);
-    vbits=64 selects the double-precision instance (the reference's -DDREAL)."""
+    """The CPU restatement.  fast=True loads the -O3 build (baseline timing), the AVX-512 one
+    where the host has it; vbits=64 selects the double-precision instance (the reference's -DDREAL)."""
 
     def __init__(self, fast=False, vbits=32):
-        self.lib = _load("libfusedmm_oracle_fast.so" if fast else "libfusedmm_oracle.so")
+        self.isa = "strict"
+        if fast:
+            self.isa = "x86-64-v3 (AVX2+FMA)"
+            name = "libfusedmm_oracle_fast.so"
+            if host_has_avx512() and os.path.exists(os.path.join(ORACLE_DIR, "libfusedmm_oracle_fast_v4.so")):
+                name, self.isa = "libfusedmm_oracle_fast_v4.so", "x86-64-v4 (AVX-512)"
+        self.lib = _load(name if fast else "libfusedmm_oracle.so")
         self.vbits = vbits
         self.np_v, self.cv = _vtype(vbits)
         self.sfx = "" if vbits == 32 else "_d"
@@ -197,22 +215,33 @@ class Oracle:
         return fn(*args)
 
 
-def _ref_name(kind, bits, vbits):
+def _ref_name(kind, bits, vbits, threads=None):
+    if threads:    # timing variant: the reference's OpenMP team fixed at `threads` (float, int32 only)
+        return "libref_%s_t%d_i%d.so" % (kind, threads, bits)
     return "libref_%s_%si%d.so" % (kind, "d_" if vbits == 64 else "", bits)
 
 
-def ref_available(kind="sigmoid", bits=32, vbits=32):
-    return os.path.exists(os.path.join(ORACLE_DIR, "_ref", _ref_name(kind, bits, vbits)))
+def ref_available(kind="sigmoid", bits=32, vbits=32, threads=None):
+    return os.path.exists(os.path.join(ORACLE_DIR, "_ref", _ref_name(kind, bits, vbits, threads)))
+
+
+REF_TIME_THREADS = (8, 16, 32, 64, 96, 128)    # TIME_THREADS of oracle/Makefile
+
+
+def ref_threads_for(cores):
+    """The largest thread count the reference's general path was built for that does not exceed `cores`."""
+    fit = [t for t in REF_TIME_THREADS if t <= max(cores, REF_TIME_THREADS[0])]
+    return fit[-1]
 
 
 class Ref:
     """The real reference (harness + generic fusedMM_csr), one library per SOP body."""
 
-    def __init__(self, kind, bits=32, vbits=32):
+    def __init__(self, kind, bits=32, vbits=32, threads=None):
         self.bits = bits
         self.np_i, self.ct = _itype(bits)
         self.np_v, self.cv = _vtype(vbits)
-        self.lib = C.CDLL(os.path.join(ORACLE_DIR, "_ref", _ref_name(kind, bits, vbits)))
+        self.lib = C.CDLL(os.path.join(ORACLE_DIR, "_ref", _ref_name(kind, bits, vbits, threads)))
         assert self.lib.ref_index_bytes() * 8 == bits and self.lib.ref_value_bytes() * 8 == vbits
 
     def table(self):

@@ -132,3 +132,90 @@ def test_cmake_target_of_the_reference_configures(tmp_path):
     if os.path.exists(exe):
         r = subprocess.run(["readelf", "-d", exe], stdout=subprocess.PIPE, text=True)
         assert "libfusedmm.so" in r.stdout
+
+
+def test_measuring_aids_are_not_in_the_product_libraries():
+    """The copy, read-stream and gather probes are the benchmark's yardsticks: they live in a library of
+    their own, and the libraries a consumer links export nothing of the kind."""
+    import subprocess
+    from fusedmm_amd import build
+    for bits in (32, 64):
+        for vbits in (32, 64):
+            syms = subprocess.run(["nm", "-D", "--defined-only", build.lib_path(bits, vbits)], stdout=subprocess.PIPE, text=True).stdout
+            assert "probe" not in syms
+            c_names = set(re.findall(r" T (\w+)$", syms, flags=re.M))
+            own = "sgfusedMM_csr" if vbits == 32 else "dgfusedMM_csr"
+            # what the library exports by a C name is exactly what the headers declare (kernel stubs aside)
+            assert {n for n in c_names if not n.startswith("_")} == set(fa.EXPORTS) | {own}
+    syms = subprocess.run(["nm", "-D", "--defined-only", build.probes_path()], stdout=subprocess.PIPE, text=True).stdout
+    assert set(re.findall(r" T (\w+)$", syms, flags=re.M)) == set(fa.PROBE_EXPORTS)
+    probes = fa.load_probes()
+    for n in fa.PROBE_EXPORTS:
+        assert hasattr(probes, n)
+    text = open(os.path.join(ROOT, "include", "fusedmm_amd.h")).read()
+    assert "probe" not in text
+
+
+_CHILD = r"""
+import ctypes as C, sys
+import numpy as np
+sys.path.insert(0, %r)
+import fusedmm_amd as fa
+lib = fa.load(32)
+%s
+"""
+
+
+def _child(body, **env):
+    import subprocess
+    import sys
+    e = dict(os.environ, **env)
+    return subprocess.run([sys.executable, "-c", _CHILD % (ROOT, body)], stdout=subprocess.PIPE, stderr=subprocess.PIPE,
+                          text=True, timeout=120, env=e)
+
+
+def test_no_usable_gpu_is_a_status_code_not_an_abort():
+    """A well-formed call (valid tuple, m > 0, host operands) in a process that sees no GPU: the HIP runtime's
+    error becomes FUSEDMM_FAIL_RETURN (reference fusedMM.h:103-112) with a message on stderr; the process goes on.
+    The condition is forced from the host (the devices are hidden from the child), so it holds on a GPU box too."""
+    body = (
+        "p = np.array([0, 2, 4], np.int32); ix = np.array([0, 1, 1, 0], np.int32)\n"
+        "v = np.ones(4, np.float32); X = np.ones((2, 8), np.float32); Z = np.zeros((2, 8), np.float32)\n"
+        "lib.fusedMM_amd_set_sop_kind(fa.SOP_KIND_SIGMOID)\n"
+        "for msg in (fa.MSG_SIGMOID, fa.MSG_GCN, fa.VOP_ADD | fa.ROP_DOT | fa.SOP_COPY | fa.VSC_MUL | fa.AOP_MAX):\n"
+        "    rc = fa.fusedMM_csr(msg, 2, 2, 8, 1.0, 4, 2, 2, v, ix, p[:-1], p[1:], X, 8, X, 8, 0.0, Z, 8)\n"
+        "    print('rc', rc)\n"
+        "print('init', lib.fusedMM_amd_init(), lib.fusedMM_amd_init_noalloc())\n"
+        "print('m0', fa.fusedMM_csr(fa.MSG_GCN, 0, 2, 8, 1.0, 4, 2, 2, v, ix, p[:-1], p[1:], X, 8, X, 8, 0.0, Z, 8))\n"
+        "print('alive', float(Z.sum()))\n")
+    r = _child(body, HIP_VISIBLE_DEVICES="", ROCR_VISIBLE_DEVICES="", CUDA_VISIBLE_DEVICES="")
+    assert r.returncode == 0, r.stderr[-2000:]
+    lines = r.stdout.split()
+    assert r.stdout.count("rc %d" % fa.FAIL) == 3, r.stdout
+    assert "init %d %d" % (fa.FAIL, fa.FAIL) in r.stdout
+    assert "m0 0" in r.stdout                          # nothing to do: success without touching any device
+    assert "alive 0.0" in r.stdout                     # Z untouched, process alive
+    assert "fusedmm_amd:" in r.stderr and "failed" in r.stderr
+
+
+def test_a_setter_overrides_the_environment_whenever_it_is_called():
+    """FUSEDMM_SPLIT / FUSEDMM_SOP_KIND are read once, by the first call into the library, whichever it is; a value
+    set through the API afterwards (also as the very first call) stays in force."""
+    body = (
+        "h, s = C.c_int64(), C.c_int()\n"
+        "%s"
+        "lib.fusedMM_amd_get_split(C.byref(h), C.byref(s)); print('split', h.value, s.value)\n"
+        "print('kind', lib.fusedMM_amd_get_sop_kind())\n")
+    env = dict(FUSEDMM_SPLIT="300,150", FUSEDMM_SOP_KIND="fr")
+    r = _child(body % "", **env)
+    assert "split 300 150" in r.stdout and "kind %d" % fa.SOP_KIND_FR in r.stdout, r.stdout + r.stderr
+    r = _child(body % "lib.fusedMM_amd_set_split(40, 20); lib.fusedMM_amd_set_sop_kind(fa.SOP_KIND_TDIST_PLAIN)\n", **env)
+    assert "split 40 20" in r.stdout and "kind %d" % fa.SOP_KIND_TDIST_PLAIN in r.stdout, r.stdout + r.stderr
+    r = _child(body % "lib.fusedMM_amd_set_split(0, 0)\n", **env)      # back to the defaults, not back to the variable
+    assert "split 0 0" in r.stdout, r.stdout
+    assert lib_rejects_unknown_kind()
+
+
+def lib_rejects_unknown_kind():
+    lib = fa.load(32)
+    return lib.fusedMM_amd_set_sop_kind(7) == -2 and lib.fusedMM_amd_set_sop_kind(-2) == -2

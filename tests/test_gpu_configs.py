@@ -101,8 +101,10 @@ class Resident:
         sub.update(rows=hi - lo, pntrb=g["pntrb"][lo:hi], pntre=g["pntre"][lo:hi])
         Xs = None if self.X is None else self.X[lo:hi]
         heavy_deg, seg_len = gpu_api.default_split(self.k)
+        # which rows are walked one per sub-wave is decided on groups of rows of the whole matrix
+        packed = gpu_api.packed_rows(g, g["rows"], self.k, 32, heavy_deg)[lo:hi]
         want = gpu_api.oracle_mirror(oracle, tkern, sub, Xs, self.Y, np.zeros((hi - lo, self.k), np.float32), 0.0, sk,
-                                     self.k, heavy_deg, seg_len)
+                                     self.k, heavy_deg, seg_len, packed=packed)
         got = Z[lo:hi].cpu().numpy()
         np.testing.assert_array_equal(got.view(np.uint32), want.view(np.uint32))
 

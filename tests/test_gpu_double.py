@@ -46,9 +46,7 @@ def test_double_pattern_ops_match_oracle(od, tkern, kind, k, bits):
     for beta in (0.0, 1.0):
         rc, Z = gpu_api.run(MSG[tkern], g, X, Y, Z0, beta=beta, bits=bits, vbits=64)
         assert rc == 0
-        V, L, S = gpu_api.layout_for(k)
-        Zw = Z0.copy()
-        od.opt("t" if tkern == "f" else tkern, g, X, Y, Zw, beta=beta, sop_kind=sk, mode=2, V=V, L=L, S=S)
+        Zw = gpu_api.oracle_mirror(od, tkern, g, X, Y, Z0, beta, sk, k, *gpu_api.default_split(k, 64), vec_ok=(k % 4 == 0))
         np.testing.assert_array_equal(Z.view(np.uint64), Zw.view(np.uint64))
     # and against the wide (long double) evaluation: double rounding only, no table flips at this size
     Zq = Z0.copy()

@@ -188,8 +188,7 @@ def test_host_arrays_allocated_exactly_as_far_as_the_reference_reads(oracle):
     rc = fa.fusedMM_csr(MSG["t"], g["rows"], g["cols"], k, 1.0, g["nnz"], g["rows"], g["cols"], g["val"], g["indx"],
                         np.ascontiguousarray(g["pntrb"]), np.ascontiguousarray(g["pntre"]), Xt, ldx, Yt, ldy, 1.0, Zt, ldz)
     assert rc == 0
-    want = Z0.copy()
-    oracle.opt("t", g, X, Y, want, beta=1.0, sop_kind=2, mode=2, V=4, L=16, S=4, k=k)
+    want = gpu_api.oracle_mirror(oracle, "t", g, X, Y, Z0, 1.0, 2, k, *gpu_api.default_split(k))
     used = (g["rows"] - 1) * ldz + k
     np.testing.assert_array_equal(np.array(Zt).view(np.uint32), want.reshape(-1)[:used].view(np.uint32))
 
@@ -243,8 +242,7 @@ def test_nan_dot_product_takes_the_first_table_bin(oracle):
     gpu_api.set_kind(SOP_NAMES["sigmoid"], 32)
     rc, Z = gpu_api.run(MSG["s"], g, X, Y, np.zeros((64, k), np.float32))
     assert rc == 0
-    want = np.zeros((64, k), np.float32)
-    oracle.opt("s", g, X, Y, want, sop_kind=1, mode=2, V=4, L=8, S=8)
+    want = gpu_api.oracle_mirror(oracle, "s", g, X, Y, np.zeros((64, k), np.float32), 0.0, 1, k, *gpu_api.default_split(k))
     np.testing.assert_array_equal(Z.view(np.uint32), want.view(np.uint32))
     assert np.isfinite(Z).all() and g["pntre"][10] > g["pntrb"][10]
     t0 = oracle.table()[0]
@@ -468,7 +466,7 @@ def test_probes_take_what_they_document(oracle):
     """The measuring aids (copy, read-stream and gather probes) run on well-formed
     arguments and refuse the rest without launching anything."""
     import torch
-    lib = fa.load(32)
+    lib = fa.load_probes()                                                  # a library of their own
     dev = torch.device("cuda:0")
     st = torch.cuda.current_stream().cuda_stream
     src = torch.arange(1 << 20, dtype=torch.float32, device=dev)            # 4 MiB

@@ -66,8 +66,7 @@ def test_m_smaller_than_rows_and_split_pointers(oracle, where):
     m = 41
     rc, Z = gpu_api.run(MSG["s"], g, X, Y, Z0, beta=0.0, bits=32, where=where, m=m)
     assert rc == 0
-    want = Z0.copy()
-    oracle.opt("s", g, X, Y, want, beta=0.0, sop_kind=1, mode=2, V=4, L=16, S=4, m=m)
+    want = gpu_api.oracle_mirror(oracle, "s", g, X, Y, Z0, 0.0, 1, k, *gpu_api.default_split(k), m=m)
     np.testing.assert_array_equal(Z.view(np.uint32), want.view(np.uint32))
     np.testing.assert_array_equal(Z[m:], Z0[m:])      # rows beyond m untouched
 
@@ -82,8 +81,7 @@ def test_leading_dimensions_larger_than_k(oracle, where):
     gpu_api.set_kind(SOP_NAMES["tdist"], 32)
     rc, Z = gpu_api.run(MSG["t"], g, X, Y, Z0, beta=1.0, bits=32, where=where, k=k)
     assert rc == 0
-    want = Z0.copy()
-    oracle.opt("t", g, X, Y, want, beta=1.0, sop_kind=2, mode=2, V=4, L=16, S=4, k=k)
+    want = gpu_api.oracle_mirror(oracle, "t", g, X, Y, Z0, 1.0, 2, k, *gpu_api.default_split(k))
     np.testing.assert_array_equal(Z.view(np.uint32), want.view(np.uint32))
     np.testing.assert_array_equal(Z[:, k:], Z0[:, k:])   # padding columns untouched
 
@@ -117,8 +115,7 @@ def test_x_and_y_are_the_same_buffer(oracle):
     rc = fa.fusedMM_csr(fa.MSG_FR, 300, 300, k, 1.0, g["nnz"], 300, 300, val, indx, pb, pe, dE, k, dE, k, 0.0, Z, k)
     assert rc == 0
     torch.cuda.synchronize()
-    want = np.zeros((300, k), np.float32)
-    oracle.opt("t", g, E, E, want, sop_kind=3, mode=2, V=4, L=8, S=8)
+    want = gpu_api.oracle_mirror(oracle, "t", g, E, E, np.zeros((300, k), np.float32), 0.0, 3, k, *gpu_api.default_split(k))
     np.testing.assert_array_equal(Z.cpu().numpy().view(np.uint32), want.view(np.uint32))
     assert np.isfinite(want).all()                    # no self loops => no 1/0
 

@@ -39,10 +39,8 @@ def test_pattern_ops_match_oracle(oracle, tkern, kind, k, bits, beta):
     gpu_api.set_kind(sk, bits)
     rc, Z = gpu_api.run(MSG[tkern], g, X, Y, Z0, beta=beta, bits=bits)
     assert rc == 0
-    V, L, S = gpu_api.layout_for(k)
     ot = "t" if tkern == "f" else tkern
-    Zw = Z0.copy()
-    oracle.opt(ot, g, X, Y, Zw, beta=beta, sop_kind=sk, mode=2, V=V, L=L, S=S)
+    Zw = gpu_api.oracle_mirror(oracle, tkern, g, X, Y, Z0, beta, sk, k, *gpu_api.default_split(k), vec_ok=(k % 4 == 0))
     np.testing.assert_array_equal(Z.view(np.uint32), Zw.view(np.uint32))
     Z64 = Z0.copy()
     oracle.opt(ot, g, X, Y, Z64, beta=beta, sop_kind=sk, mode=1)
@@ -64,7 +62,5 @@ def test_host_operands(oracle, tkern, kind, bits):
     gpu_api.set_kind(sk, bits)
     rc, Z = gpu_api.run(MSG[tkern], g, X, Y, Z0, beta=0.0, bits=bits, where="host")
     assert rc == 0
-    V, L, S = gpu_api.layout_for(k)
-    Zw = Z0.copy()
-    oracle.opt("t" if tkern == "f" else tkern, g, X, Y, Zw, beta=0.0, sop_kind=sk, mode=2, V=V, L=L, S=S)
+    Zw = gpu_api.oracle_mirror(oracle, tkern, g, X, Y, Z0, 0.0, sk, k, *gpu_api.default_split(k))
     np.testing.assert_array_equal(Z.view(np.uint32), Zw.view(np.uint32))

@@ -6,7 +6,7 @@ import pytest
 import scipy.sparse as sp
 
 import graphs
-from oracle_api import MSG, SOP_FR, SOP_SIGMOID, SOP_TDIST, SOP_LL, SOP_FA
+from oracle_api import MSG, SOP_FR, SOP_SIGMOID, SOP_TDIST, SOP_LL, SOP_FA, SOP_TDIST_PLAIN
 
 
 def _csr_matrix(g, pattern=False):
@@ -96,12 +96,13 @@ def _dense_brute(tkern, kind, table, g, X, Y):
             else:
                 d = X64[i] - Y64[c]
                 s = float(np.float32(d @ d))
-                w = {"tdist": max(-5.0, min(5.0, -2.0 / (1.0 + s))), "fr": 1.0 + 1.0 / s}[kind]
+                w = {"tdist": max(-5.0, min(5.0, -2.0 / (1.0 + s))), "fr": 1.0 + 1.0 / s, "tdist_plain": 1.0 / (1.0 + s)}[kind]
                 Z[i] += w * d
     return Z
 
 
-@pytest.mark.parametrize("tkern,kind,sk", [("s", "sigmoid", SOP_SIGMOID), ("t", "tdist", SOP_TDIST), ("t", "fr", SOP_FR)])
+@pytest.mark.parametrize("tkern,kind,sk", [("s", "sigmoid", SOP_SIGMOID), ("t", "tdist", SOP_TDIST), ("t", "fr", SOP_FR),
+                                           ("t", "tdist_plain", SOP_TDIST_PLAIN)])
 def test_embedding_ops_equal_dense_brute_force(oracle, tkern, kind, sk):
     g = graphs.tiny_er(60, 200, seed=5)
     k = 16
@@ -132,6 +133,48 @@ def test_sigmoid_special_cases(oracle):
     Z = np.zeros((g["rows"], k), np.float32)
     oracle.opt("s", g, -Xpos, Ybig, Z, sop_kind=SOP_SIGMOID)
     np.testing.assert_allclose(Z, _csr_matrix(g, True) @ Ybig.astype(np.float64), rtol=1e-5)
+
+
+@pytest.mark.parametrize("vbits", [32, 64])
+def test_plain_tdist_weight_is_pinned_by_its_closed_form_and_by_the_harness_body(vbits):
+    """1/(1+s), the t-distribution weight as written in the benchmark list; no body of the reference's tester
+    computes it.  Exact values on arguments where 1/(1+s) is a power of two; the exact relation -2 * plain ==
+    the tester's t-dist body (bit for bit: scaling by a power of two commutes with the one rounding, and the
+    body's clamp to [-5, 5] never binds for s >= 0); monotone, in (0, 1]; a plausible slip (1/s, 1/(1+s)^2,
+    a missing 1, float instead of double arithmetic) fails one of these."""
+    from oracle_api import Oracle
+    o = Oracle(vbits=vbits)
+    npv = np.float32 if vbits == 32 else np.float64
+    s = np.array([0.0, 1.0, 3.0, 7.0, 1023.0, 0.5, 0.25], npv)
+    np.testing.assert_array_equal(o.sop(SOP_TDIST_PLAIN, s), np.array([1, 0.5, 0.25, 0.125, 1.0 / 1024, 1 / 1.5, 0.8], npv))
+    rng = np.random.Generator(np.random.Philox(key=[4, 4]))
+    v = np.concatenate([rng.uniform(0, 40, 5000), rng.uniform(0, 1e-3, 500), 10.0 ** rng.uniform(2, 30, 500)]).astype(npv)
+    plain, body = o.sop(SOP_TDIST_PLAIN, v), o.sop(SOP_TDIST, v)
+    np.testing.assert_array_equal((npv(-2) * plain).view(np.uint32 if vbits == 32 else np.uint64),
+                                  body.view(np.uint32 if vbits == 32 else np.uint64))
+    assert (plain > 0).all() and (plain <= 1).all()
+    order = np.argsort(v, kind="stable")
+    assert (np.diff(plain[order]) <= 0).all()
+    # one rounding of the double-precision quotient (what the tester's conventions give), not float arithmetic
+    want = (1.0 / (1.0 + v.astype(np.float64))).astype(npv)
+    np.testing.assert_array_equal(plain, want)
+
+
+def test_plain_tdist_identical_rows_contribute_nothing(oracle):
+    g = graphs.tiny_er(40, 100, seed=7)
+    k = 8
+    Y = np.tile(graphs.features(1, k, 3), (g["cols"], 1))
+    Z = np.zeros((g["rows"], k), np.float32)
+    oracle.opt("t", g, Y.copy(), Y, Z, sop_kind=SOP_TDIST_PLAIN)
+    assert not Z.any()                                         # weight 1, difference 0
+    # and the whole op is -1/2 of the tester's t-dist op, term by term (mode 0: multiply and add rounded
+    # separately, so the factor -2 stays exact through every step)
+    X = graphs.features(g["rows"], k, 5, -1, 1)
+    Yr = graphs.features(g["cols"], k, 6, -1, 1, stream=2)
+    Za, Zb = np.zeros((g["rows"], k), np.float32), np.zeros((g["rows"], k), np.float32)
+    oracle.opt("t", g, X, Yr, Za, sop_kind=SOP_TDIST_PLAIN)
+    oracle.opt("t", g, X, Yr, Zb, sop_kind=SOP_TDIST)
+    np.testing.assert_array_equal((np.float32(-2) * Za).view(np.uint32), Zb.view(np.uint32))
 
 
 def test_tdist_identical_rows_and_fr_nan(oracle):
