@@ -30,6 +30,14 @@ FLAGS = [
     # well (-Xarch_device takes no option with an argument), which answers with the line filtered below.
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
 ]
+# experiments: FUSEDMM_BUILD_EXTRA="-DX=1 ..." adds compiler flags, FUSEDMM_BUILD_OUT=<dir> writes libraries and
+# objects there (load them with FUSEDMM_AMD_LIB_DIR=<dir>)
+FLAGS += os.environ.get("FUSEDMM_BUILD_EXTRA", "").split()
+if os.environ.get("FUSEDMM_BUILD_OUT"):
+    OUT = os.path.abspath(os.environ["FUSEDMM_BUILD_OUT"])
+    OBJ = os.path.join(OUT, "obj")
+else:
+    OUT = HERE
 HOST_PASS_NOISE = "'-packed-fp32-ops' is not a recognized feature for this target (ignoring feature)"
 
 # translation units of a product library: (source, extra defines, object tag)
@@ -54,7 +62,8 @@ def lib_path(index_bits, value_bits=32):
 
 
 def probes_path():
-    return os.path.join(os.environ.get("FUSEDMM_AMD_LIB_DIR", HERE), "libfusedmm_amd_probes.so")
+    p = os.path.join(os.environ.get("FUSEDMM_AMD_LIB_DIR", HERE), "libfusedmm_amd_probes.so")
+    return p if os.path.exists(p) else os.path.join(HERE, "libfusedmm_amd_probes.so")
 
 
 def variant_defines(index_bits, value_bits):
@@ -119,9 +128,9 @@ def build_libs(variants=VARIANTS, force=False, verbose=False, probes=True):
         list(ex.map(lambda j: _compile(j[0], j[1], j[2], force, verbose), jobs))
     libs = []
     for ib, vb in variants:
-        libs.append(_link(os.path.join(HERE, lib_name(ib, vb)), [o for _, o, _ in _objects(ib, vb)], verbose, ["-ldl"]))
+        libs.append(_link(os.path.join(OUT, lib_name(ib, vb)), [o for _, o, _ in _objects(ib, vb)], verbose, ["-ldl"]))
     if probes:
-        libs.append(_link(os.path.join(HERE, "libfusedmm_amd_probes.so"), [os.path.join(OBJ, "probes.o")], verbose))
+        libs.append(_link(os.path.join(OUT, "libfusedmm_amd_probes.so"), [os.path.join(OBJ, "probes.o")], verbose))
     return libs
 
 

@@ -19,6 +19,17 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+// ---- A/B switches of one-off experiments (all off by default) ----
+#ifndef FMM_AB_L64_VECTOR
+#define FMM_AB_L64_VECTOR 0      // 1: whole-wave rows take column ids through ds_bpermute into vector registers
+#endif
+#ifndef FMM_AB_Z_PLAIN_STORE
+#define FMM_AB_Z_PLAIN_STORE 0   // 1: finished Z rows are stored with plain (write-back) stores
+#endif
+#ifndef FMM_AB_EARLY_ROWS
+#define FMM_AB_EARLY_ROWS 0      // n > 0: one wave in n skips the segment phase and starts on rows at once
+#endif
+
 namespace fmm {
 
 // The library is compiled once per value type, as the reference is (-DDREAL).
@@ -206,20 +217,27 @@ __device__ __forceinline__ real_t cross_subwave_sum(real_t v)
    if (L <= 32) v = add_xor32(v);
    return v;
 }
+// MAX and MIN of the accumulate stage across sub-waves.  The reference's fmax / fmin are the ternaries
+// (x) > (y) ? (x) : (y) and (x) < (y) ? (x) : (y) (fusedMM.c:18-19): a NaN on the left loses, a NaN on the
+// right wins, so what a row with a NaN term comes to depends on the order of its edges.  Here a sub-wave
+// folds its own edges with that very ternary, in edge order; where accumulators are combined a NaN is kept
+// (both lanes of a pair then agree, and a row with a single edge gives exactly the reference's result).
+__device__ __forceinline__ real_t merge_max(real_t v, real_t o) { const real_t r = max_r(v, o); return v != v ? v : r; }
+__device__ __forceinline__ real_t merge_min(real_t v, real_t o) { const real_t r = min_r(v, o); return v != v ? v : r; }
 template <int L>
 __device__ __forceinline__ real_t cross_subwave_max(real_t v)
 {
-   if (L <= 8) v = max_r(v, dpp<0x128>(v));
-   if (L <= 16) v = max_r(v, lane_xor16(v));
-   if (L <= 32) v = max_r(v, (real_t)__shfl_xor(v, 32, 64));
+   if (L <= 8) v = merge_max(v, dpp<0x128>(v));
+   if (L <= 16) v = merge_max(v, lane_xor16(v));
+   if (L <= 32) v = merge_max(v, (real_t)__shfl_xor(v, 32, 64));
    return v;
 }
 template <int L>
 __device__ __forceinline__ real_t cross_subwave_min(real_t v)
 {
-   if (L <= 8) v = min_r(v, dpp<0x128>(v));
-   if (L <= 16) v = min_r(v, lane_xor16(v));
-   if (L <= 32) v = min_r(v, (real_t)__shfl_xor(v, 32, 64));
+   if (L <= 8) v = merge_min(v, dpp<0x128>(v));
+   if (L <= 16) v = merge_min(v, lane_xor16(v));
+   if (L <= 32) v = merge_min(v, (real_t)__shfl_xor(v, 32, 64));
    return v;
 }
 
@@ -743,7 +761,7 @@ __device__ __forceinline__ void load_chunk(EdgeChunk<IdxT> &c, const Params<IdxT
 template <int L>
 __device__ __forceinline__ int32_t chunk_entry(int32_t v, int e)
 {
-   if (L == 64) return __builtin_amdgcn_readlane(v, e);
+   if (L == 64 && !FMM_AB_L64_VECTOR) return __builtin_amdgcn_readlane(v, e);
    return __builtin_amdgcn_ds_bpermute(e << 2, v);
 }
 template <int L>
@@ -1305,8 +1323,17 @@ __device__ __forceinline__ void segments_phase(const Params<IdxT> &p, lds_table_
 
    const int lane = threadIdx.x & 63;
    const int sub = lane / L, sl = lane % L;
+#if FMM_AB_EARLY_ROWS > 0
+   const int64_t w_all = (int64_t)blockIdx.x * kWavesPerBlock + (threadIdx.x >> 6);
+   const int64_t n_all = (int64_t)gridDim.x * kWavesPerBlock;
+   constexpr int64_t kN = FMM_AB_EARLY_ROWS;
+   if (n_all >= 2 * kN && w_all % kN == kN - 1) return;                    // this wave starts on rows at once
+   const int64_t wave0 = n_all >= 2 * kN ? (kN - 1) * (w_all / kN) + w_all % kN : w_all;
+   const int64_t nwaves = n_all >= 2 * kN ? (n_all / kN) * (kN - 1) + ((n_all % kN) < (kN - 1) ? (n_all % kN) : (kN - 1)) : n_all;
+#else
    const int64_t wave0 = (int64_t)blockIdx.x * kWavesPerBlock + (threadIdx.x >> 6);
    const int64_t nwaves = (int64_t)gridDim.x * kWavesPerBlock;
+#endif
    const bool reads_x = op_reads_x<OP>(p.imessage);
    const int aop = p.imessage & 0xF0000;
 
@@ -1539,7 +1566,7 @@ __device__ __forceinline__ void rows_phase(const Params<IdxT> &p, lds_table_t ta
             load_slice<V, L, R, EXACT>(zin, zrow, sl, p.k);
             map2(acc, zin, acc, [](real_t a, real_t b) { return a + b; });
          }
-         store_slice<V, L, R, EXACT, true>(zrow, acc, sl, p.k);
+         store_slice<V, L, R, EXACT, !FMM_AB_Z_PLAIN_STORE>(zrow, acc, sl, p.k);
       }
    }
    chunk = nc > 0 ? resolve_claim<IdxT>(p, claimed, cur, nc, nchunks, lane) : -1;

@@ -91,6 +91,10 @@ void fusedMM_amd_set_stage_callbacks(fusedMM_amd_vop_fn vop, fusedMM_amd_rop_fn 
  * call of the same size before capturing; a later, larger call re-allocates the
  * queues and invalidates graphs captured earlier (fusedMM_csr_stream_noalloc has
  * neither restriction).
+ * A stream that carried an eager call must not
+ * enter a capture while a call on ANOTHER stream may still have to be ordered after it: that
+ * call is refused with FUSEDMM_FAIL_RETURN (an event recorded on a capturing stream would
+ * become a node of the caller's graph), and succeeds once the capture has ended.
  * FUSEDMM_SOP_KIND_HOST is
  * not available here (it needs the host between passes): returns
  * FUSEDMM_UNDEFINED_USER_FUNCTION.

@@ -19,6 +19,9 @@ full so nothing has to be regenerated bit-for-bit) and the reference's outputs:
                       evaluated each row on, for the degree sets of
                       graphs.partition_cases() (-1: a row without edges, whose
                       holder the reference never shows)
+  special_values.npz  Z of the reference's fusedMM_csr (general pipeline) for the MAX / MIN
+                      tuples on operands salted with NaN, infinities and zeros of both signs
+                      (graphs.special_values_case), float and (keys ending in _d) double
   udef_stages.npz     Z of the reference's fusedMM_csr built with VOP/ROP/VSC/
                       AOP_UDEF_IMPL switched on and linked with the caller-side
                       stage functions of oracle/udef_stage_bodies.inc, for op
@@ -166,6 +169,20 @@ def main():
             out["%s_owner_t%d" % (name, t)] = own32.astype(np.int8)
     out["names"] = np.array(names)
     np.savez_compressed(os.path.join(HERE, "partition.npz"), **out)
+
+    # MAX / MIN stages on NaN, infinities and signed zeros
+    multi, single, X, Y, Z0, msgs = graphs.special_values_case(32)
+    out = {"msgs": msgs}
+    for sfx, vbits, npv in (("", 32, np.float32), ("_d", 64, np.float64)):
+        r = Ref("tdist", 32, vbits)
+        for gname, g in (("multi", multi), ("single", single)):
+            Zs = np.zeros((len(msgs),) + Z0.shape, npv)
+            for n, imsg in enumerate(msgs):
+                Z = Z0.astype(npv)
+                assert r.fusedMM_csr(int(imsg), g, X.astype(npv), Y.astype(npv), Z) == 0
+                Zs[n] = Z
+            out["Z_%s%s" % (gname, sfx)] = Zs
+    np.savez_compressed(os.path.join(HERE, "special_values.npz"), **out)
 
     # tuples with user stages through the reference built with those stages switched on
     g = graphs.with_values(graphs.ragged(32, rows=37, cols=53, hub_deg=90))

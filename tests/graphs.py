@@ -176,3 +176,35 @@ def boundary_graph(bits=32, cols=500, seed=21):
     g = synth.graph_from_rowptr(deg.size, cols, rowptr, indx, None, bits)
     g["val"] = synth.edge_values(g["nnz"], seed)
     return g
+
+
+def special_values_case(bits=32, seed=31):
+    """Inputs with NaN, infinities and zeros of both signs, for the MAX / MIN stages (the reference's own
+    fmax / fmin are the ternaries (x) > (y) ? (x) : (y) and (x) < (y) ? (x) : (y), fusedMM.c:18-19, so a NaN
+    on the left loses and a NaN on the right wins, and of two zeros the right one is kept).  Two graphs over
+    the same operands: `multi` with ordinary rows (the order of edges matters once a NaN is involved) and
+    `single` with at most one edge per row (no order to depend on).  Returns (multi, single, X, Y, Z0, tuples)."""
+    rng = np.random.Generator(np.random.Philox(key=[seed, 0]))
+    rows, cols, k = 40, 30, 8
+    multi = ragged(bits, seed=seed, rows=rows, cols=cols, hub_deg=50)
+    deg1 = (rng.random(rows) < 0.8).astype(np.int64)
+    rowptr = np.zeros(rows + 1, np.int64)
+    np.cumsum(deg1, out=rowptr[1:])
+    single = synth.graph_from_rowptr(rows, cols, rowptr, rng.integers(0, cols, int(rowptr[-1]), dtype=np.int64), None, bits)
+    single["val"] = synth.edge_values(single["nnz"], seed)
+    special = np.array([np.nan, -0.0, 0.0, np.inf, -np.inf, 1.0, -1.0], np.float32)
+
+    def salted(n, stream):
+        a = features(n, k, seed, -1, 1, stream)
+        hit = rng.random((n, k)) < 0.35
+        a[hit] = special[rng.integers(0, special.size, int(hit.sum()))]
+        return a
+    X, Y, Z0 = salted(rows, 1), salted(cols, 2), salted(rows, 3)
+    tuples = []
+    for vop in (0x6, 0x7, 0x2):                    # VOP_MAX, VOP_MIN, VOP_COPY_RHS
+        for aop in (0x10000, 0x20000, 0x30000):    # AOP_ADD, AOP_MAX, AOP_MIN
+            if vop == 0x2 and aop == 0x10000:
+                continue
+            tuples.append(vop | 0x00 | 0x000 | 0x0000 | aop)        # ROP_NOOP, SOP_NOOP, VSC_NOOP: T goes straight to AOP
+            tuples.append(vop | 0x30 | 0x100 | 0x1000 | aop)        # ROP_ADD_RHS, SOP_COPY, VSC_MUL
+    return multi, single, X, Y, Z0, np.array(tuples, np.int32)

@@ -370,6 +370,45 @@ def test_capture_refuses_what_would_block(oracle):
         assert torch.equal(Z1, Zeager) and torch.equal(Z2, Zeager), rep
 
 
+def test_a_call_is_not_ordered_after_a_stream_that_entered_capture(oracle):
+    """Calls on different streams are ordered by an event recorded on the earlier call's stream.  When that
+    stream has meanwhile entered a capture, such a record would become a node of the caller's graph: the new call
+    is refused (FUSEDMM_FAIL_RETURN, nothing enqueued, no device-wide wait), the capture stays valid, and the
+    same call goes through once the capture has ended."""
+    import torch
+    lib = fa.load(64)
+    assert lib.fusedMM_amd_init() == 0
+    g = graphs.with_values(graphs.tiny_er(300, 2000, 22, bits=64))
+    k = 32
+    Y = graphs.features(300, k, 6, -0.5, 0.5, 2)
+    d = dict(val=_dev(g["val"]), indx=_dev(g["indx"]), pb=_dev(g["pntrb"]), pe=_dev(g["pntre"]), Y=_dev(Y))
+    dev = torch.device("cuda:0")
+
+    def enqueue(Z, stream):
+        return fa.fusedMM_csr(fa.MSG_SPMM, g["rows"], g["cols"], k, 1.0, g["nnz"], g["rows"], g["cols"], d["val"], d["indx"],
+                              d["pb"], d["pe"], None, k, d["Y"], k, 0.0, Z, k, index_bits=64, stream=stream.cuda_stream)
+
+    s1, s2 = torch.cuda.Stream(), torch.cuda.Stream()
+    Za = torch.zeros((g["rows"], k), device=dev)
+    Zb = torch.full((g["rows"], k), 5.0, device=dev)
+    Zw = torch.zeros(16, device=dev)
+    torch.cuda.synchronize()
+    assert enqueue(Za, s1) == 0                                # eager, on s1: the queues' last user
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph, stream=s1):                   # s1 enters a capture
+        Zw.add_(1.0)
+        rc_refused = enqueue(Zb, s2)                           # would have to record an event on s1
+    assert rc_refused == fa.FAIL
+    torch.cuda.synchronize()
+    assert float(Zb.min()) == 5.0 and float(Zb.max()) == 5.0   # nothing ran
+    graph.replay()                                             # the capture was left intact
+    torch.cuda.synchronize()
+    assert float(Zw.sum()) == 16.0
+    assert enqueue(Zb, s2) == 0                                # the capture has ended: ordered and run
+    torch.cuda.synchronize()
+    assert torch.equal(Za, Zb) and float(Za.abs().max()) > 0
+
+
 def test_capture_never_reallocates_work_queues(oracle):
     """Under HIP graph capture fusedMM_csr_stream refuses a call whose work queues
     would have to grow (replacing them would leave earlier graphs with freed

@@ -284,3 +284,43 @@ def test_finalize_releases_and_the_library_recovers(oracle):
     rc, Zb = gpu_api.run(MSG["s"], g, X, Y, Z0, where="host")
     assert rc == 0
     np.testing.assert_array_equal(Za.view(np.uint32), Zb.view(np.uint32))
+
+
+def _same_special(Z, want, imsg, u, what):
+    """NaN for NaN; elsewhere the same bits -- except where the tuple sums over the row's elements (a ROP), whose
+    order differs between the wavefront and the reference's loop: there, infinities equal and the rest to rounding."""
+    nz, nw = np.isnan(Z), np.isnan(want)
+    np.testing.assert_array_equal(nz, nw, err_msg=what)
+    if (imsg & 0xF0) == 0:
+        np.testing.assert_array_equal(Z.view(u)[~nz], want.view(u)[~nw], err_msg=what)
+    else:
+        np.testing.assert_allclose(Z[~nz], want[~nw], rtol=1e-5, atol=1e-6, err_msg=what)
+
+
+@pytest.mark.parametrize("where", ["device", "host"])
+@pytest.mark.parametrize("bits,vbits", [(32, 32), (64, 32), (32, 64)])
+def test_max_and_min_stages_on_nan_and_signed_zeros_match_the_reference(where, bits, vbits):
+    """VOP_MAX / VOP_MIN / AOP_MAX / AOP_MIN on operands salted with NaN, infinities and zeros of both signs,
+    rows with at most one edge (with more, what a NaN term leaves behind depends on the order of the edges,
+    in the reference as here): the reference's own output, NaN for NaN and bit for bit elsewhere.  Its fmax /
+    fmin are the ternaries of fusedMM.c:18-19 -- a NaN on the right wins, the right one of two zeros is kept --
+    and so are the kernels'; where sub-wave accumulators are combined a NaN is kept."""
+    import os
+    d = np.load(os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "special_values.npz"))
+    multi, single, X, Y, Z0, msgs = graphs.special_values_case(bits)
+    npv, sfx, u = (np.float32, "", np.uint32) if vbits == 32 else (np.float64, "_d", np.uint64)
+    for imsg, want in zip(msgs, d["Z_single" + sfx]):
+        rc, Z = gpu_api.run(int(imsg), single, X.astype(npv), Y.astype(npv), Z0.astype(npv), bits=bits, vbits=vbits, where=where)
+        assert rc == 0
+        _same_special(Z, want, int(imsg), u, hex(int(imsg)))
+    # the same operands with the packing of short rows switched off: every row goes through the merge of
+    # the sub-wave accumulators, which must keep what the single edge left
+    lib = fa.load(bits, vbits)
+    prev = lib.fusedMM_amd_set_pack_rows(0)
+    try:
+        for imsg, want in zip(msgs, d["Z_single" + sfx]):
+            rc, Z = gpu_api.run(int(imsg), single, X.astype(npv), Y.astype(npv), Z0.astype(npv), bits=bits, vbits=vbits, where=where)
+            assert rc == 0
+            _same_special(Z, want, int(imsg), u, "unpacked " + hex(int(imsg)))
+    finally:
+        lib.fusedMM_amd_set_pack_rows(prev)

@@ -37,7 +37,8 @@ def test_plain_tdist_body_on_the_device(k, bits, vbits):
         gpu_api.set_kind(fa.SOP_KIND_TDIST, bits, vbits)
         rc, Zt = gpu_api.run(MSG["t"], g, X, Y, Z0, beta=0.0, bits=bits, vbits=vbits)
         assert rc == 0
-        np.testing.assert_array_equal((npv(-2) * Zp).view(ubits), Zt.view(ubits))
+        # (+ 0: the empty rows' zeros come out of the multiplication with the other sign)
+        np.testing.assert_array_equal((npv(-2) * Zp + npv(0)).view(ubits), (Zt + npv(0)).view(ubits))
         # closed form in double precision from the definition
         deg = (g["pntre"] - g["pntrb"]).astype(np.int64)
         Zd = np.zeros((g["rows"], k))
@@ -97,7 +98,7 @@ def test_host_function_stages_over_a_window_high_in_the_arrays(where):
     X = graphs.features(g["rows"], k, 5, -1, 1, 1)
     Y = graphs.features(g["cols"], k, 5, -1, 1, 2)
     Z0 = graphs.features(g["rows"], k, 5, -1, 1, 3)
-    lo, hi = 231, 297
+    lo, hi = 232, 296      # whole groups of 8 rows: which short rows share a wavefront is decided per such group
     assert g["pntrb"][lo] > 0.5 * g["nnz"]
     sub = dict(g)
     sub.update(rows=hi - lo, pntrb=np.ascontiguousarray(g["pntrb"][lo:hi]), pntre=np.ascontiguousarray(g["pntre"][lo:hi]))

@@ -3,6 +3,8 @@
 import os
 
 import numpy as np
+
+import graphs
 import pytest
 
 from oracle_api import MSG, SOP_NAMES
@@ -227,3 +229,34 @@ def test_user_stage_without_a_function_is_undefined(oracle):
         Z = Z0.copy()
         assert oracle.generic(imsg, g, X, Y, Z) == 64
         np.testing.assert_array_equal(Z, Z0)
+
+
+def same_values(a, b):
+    """NaN in the same places, the same bits everywhere else (so a zero's sign counts)."""
+    a, b = np.asarray(a), np.asarray(b)
+    u = np.uint32 if a.dtype == np.float32 else np.uint64
+    na, nb = np.isnan(a), np.isnan(b)
+    return a.dtype == b.dtype and np.array_equal(na, nb) and np.array_equal(a.view(u)[~na], b.view(u)[~nb])
+
+
+@pytest.mark.parametrize("vbits", [32, 64])
+def test_max_and_min_stages_on_nan_infinities_and_signed_zeros(oracle, oracle_d, vbits):
+    """The reference's fmax / fmin are macros, (x) > (y) ? (x) : (y) and (x) < (y) ? (x) : (y) (fusedMM.c:18-19),
+    not the C library's: a NaN on the left loses, on the right wins; of two zeros the right one is kept.  The
+    oracle's VOP_MAX / VOP_MIN / AOP_MAX / AOP_MIN against the real reference's output on such operands."""
+    d = np.load(os.path.join(GOLD, "special_values.npz"))
+    multi, single, X, Y, Z0, msgs = graphs.special_values_case(32)
+    o, npv, sfx = (oracle, np.float32, "") if vbits == 32 else (oracle_d, np.float64, "_d")
+    assert np.array_equal(msgs, d["msgs"]) and np.isnan(X).any() and np.signbit(Y[Y == 0]).any()
+    seen_nan = seen_negzero = 0
+    for gname, g in (("multi", multi), ("single", single)):
+        for imsg, want in zip(msgs, d["Z_%s%s" % (gname, sfx)]):
+            Z = Z0.astype(npv)
+            assert o.generic(int(imsg), g, X.astype(npv), Y.astype(npv), Z) == 0
+            assert same_values(Z, want), (gname, hex(int(imsg)))
+            seen_nan += int(np.isnan(want).sum())
+            seen_negzero += int((np.signbit(want) & (want == 0)).sum())
+    assert seen_nan > 100 and seen_negzero > 20
+    # the C library's fmax / fmin would differ on these operands (it never returns the NaN of a pair)
+    a, b = np.float32(1.0), np.float32(np.nan)
+    assert np.isnan(a if a > b else b) and not np.isnan(np.fmax(a, b))

@@ -129,3 +129,23 @@ def test_user_stage_tuples_live(bits, vbits):
         assert np.array_equal(za.view(np.uint8), zb.view(np.uint8)), hex(msg)
         n += 1
     assert n == 1344
+
+
+@pytest.mark.parametrize("vbits", [32, 64])
+def test_max_min_on_special_values_live(vbits):
+    """Fresh operands with NaN, infinities and signed zeros through the real reference's general pipeline and
+    the oracle's: NaN for NaN, bit for bit elsewhere (the committed vectors are tests/golden/special_values.npz)."""
+    from oracle_api import Oracle, Ref, ref_available
+    if not ref_available("tdist", 32, vbits):
+        pytest.skip("oracle/_ref not built")
+    npv, u = (np.float32, np.uint32) if vbits == 32 else (np.float64, np.uint64)
+    o, r = Oracle(vbits=vbits), Ref("tdist", 32, vbits)
+    for seed in (41, 42, 43):
+        multi, single, X, Y, Z0, msgs = graphs.special_values_case(32, seed)
+        for g in (multi, single):
+            for imsg in msgs:
+                Za, Zb = Z0.astype(npv), Z0.astype(npv)
+                assert o.generic(int(imsg), g, X.astype(npv), Y.astype(npv), Za) == 0
+                assert r.fusedMM_csr(int(imsg), g, X.astype(npv), Y.astype(npv), Zb) == 0
+                na, nb = np.isnan(Za), np.isnan(Zb)
+                assert np.array_equal(na, nb) and np.array_equal(Za.view(u)[~na], Zb.view(u)[~nb]), (seed, hex(int(imsg)))

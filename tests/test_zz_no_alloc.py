@@ -126,3 +126,58 @@ def test_sizes_beyond_the_array_are_refused_and_touch_nothing():
     Zw = dw["Z0"].clone()
     assert _call(fa.MSG_SPMM, g, dw, kw, 0.0, Zw, 32, 32, True) == fa.NOT_ENOUGH_MEM
     assert not bool(Zw.any())
+
+
+def test_calls_leave_device_memory_as_they_found_it_and_match_the_oracle():
+    """The property the entry point exists for: after the set-up call that allocates nothing either
+    (fusedMM_amd_init_noalloc) and one warm-up call, a series of calls of different sizes, ops and K -- one of
+    them splitting rows -- changes the free device memory by not one byte.  Run on a library whose grown queues
+    were released (fusedMM_amd_finalize), so that a fall-back to the growing path would show as an allocation.
+    One of the results is also held to the CPU oracle's mirror of the kernels, bit for bit."""
+    import torch
+    from oracle_api import Oracle
+    lib = fa.load(32)
+    # (the static array is part of the library's code object: it comes into being when the runtime loads that
+    # object, on the library's first use in the process -- make sure that lies behind us)
+    assert lib.fusedMM_amd_init_noalloc() == 0
+    torch.cuda.synchronize()
+    lib.fusedMM_amd_finalize()                       # nothing grown is left; the static array stays (it is not an allocation)
+    free0 = torch.cuda.mem_get_info()[0]
+    assert lib.fusedMM_amd_init_noalloc() == 0
+    torch.cuda.synchronize()
+    assert torch.cuda.mem_get_info()[0] == free0     # the set-up call allocated no device memory
+
+    cases = []
+    g1 = graphs.with_values(graphs.tiny_er(3000, 20000, 5))
+    cases.append(("s", fa.MSG_SIGMOID, 1, g1, graphs.features(3000, 128, 3, -0.5, 0.5, 1), graphs.features(3000, 128, 3, -0.5, 0.5, 2), 0.0))
+    g2 = graphs.ragged(32, rows=64, cols=5000, hub_deg=40000)      # its hub row is cut into segments
+    cases.append(("m", fa.MSG_SPMM, 0, g2, None, graphs.features(5000, 64, 2, -0.5, 0.5, 2), 1.0))
+    g3 = graphs.boundary_graph()                                      # short rows, walked one per sub-wave
+    cases.append(("t", fa.MSG_TDIST, 2, g3, graphs.features(g3["rows"], 32, 4, -1, 1, 1), graphs.features(g3["cols"], 32, 4, -1, 1, 2), 0.0))
+    g4 = graphs.ragged(32, hub_deg=300)
+    cases.append(("g", fa.MSG_GCN, 0, g4, None, graphs.features(g4["cols"], 512, 6, -0.5, 0.5, 2), 0.0))
+    ops = []
+    for tkern, imsg, sk, g, X, Y, beta in cases:      # every operand resident before the measurement starts
+        Z0 = graphs.features(g["rows"], Y.shape[1], 9, -1, 1, 3)
+        ops.append((tkern, imsg, sk, g, X, Y, Z0, beta, _device_operands(g, X, Y, Z0)))
+    outs = [o[8]["Z0"].clone() for o in ops]
+    # warm-up (module loading, first launch of each kernel instance), then the measured series
+    for (tkern, imsg, sk, g, X, Y, Z0, beta, d), Z in zip(ops, outs):
+        gpu_api.set_kind(sk)
+        assert _call(imsg, g, d, Y.shape[1], beta, Z, 32, 32, True) == 0
+    torch.cuda.synchronize()
+    free1 = torch.cuda.mem_get_info()[0]
+    for rep in range(3):
+        for (tkern, imsg, sk, g, X, Y, Z0, beta, d), Z in zip(ops, outs):
+            Z.copy_(d["Z0"])
+            gpu_api.set_kind(sk)
+            assert _call(imsg, g, d, Y.shape[1], beta, Z, 32, 32, True) == 0
+            if tkern == "m":
+                assert gpu_api.last_split()[1] > 1
+    torch.cuda.synchronize()
+    assert torch.cuda.mem_get_info()[0] == free1      # not one byte allocated or freed by twelve calls
+    oracle = Oracle()
+    for (tkern, imsg, sk, g, X, Y, Z0, beta, d), Z in zip(ops, outs):
+        k = Y.shape[1]
+        want = gpu_api.oracle_mirror(oracle, tkern, g, X, Y, Z0, beta, sk, k, *gpu_api.default_split(k))
+        np.testing.assert_array_equal(Z.cpu().numpy().view(np.uint32), want.view(np.uint32), err_msg=tkern)
