@@ -213,13 +213,10 @@ int launch_zero_rows(val_t *z, int64_t m, int64_t k, int64_t ldz, int num_cu, hi
 #else
 #define FMM_U(u) (u)
 #endif
-#ifndef FMM_AB_U256
-#define FMM_AB_U256 16
-#endif
 #define FMM_SHAPES(X) \
-   X(4, 8, 1, 1, FMM_U(8)) X(4, 16, 1, 1, FMM_U(8)) X(4, 32, 1, 1, FMM_U(8)) X(4, 64, 1, 1, FMM_U(FMM_AB_U256)) \
+   X(4, 8, 1, 1, FMM_U(8)) X(4, 16, 1, 1, FMM_U(8)) X(4, 32, 1, 1, FMM_U(8)) X(4, 64, 1, 1, FMM_U(16)) \
    X(4, 64, 2, 1, FMM_U(8)) \
-   X(4, 8, 1, 0, FMM_U(8)) X(4, 16, 1, 0, FMM_U(8)) X(4, 32, 1, 0, FMM_U(8)) X(4, 64, 1, 0, FMM_U(FMM_AB_U256)) \
+   X(4, 8, 1, 0, FMM_U(8)) X(4, 16, 1, 0, FMM_U(8)) X(4, 32, 1, 0, FMM_U(8)) X(4, 64, 1, 0, FMM_U(16)) \
    X(4, 64, 2, 0, FMM_U(8)) X(4, 64, 4, 0, FMM_U(4)) X(4, 64, 8, 0, FMM_U(2)) \
    X(1, 64, 1, 0, FMM_U(16)) X(1, 64, 2, 0, FMM_U(8)) X(1, 64, 4, 0, FMM_U(4)) X(1, 64, 8, 0, FMM_U(2))
 

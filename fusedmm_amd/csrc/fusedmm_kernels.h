@@ -19,17 +19,6 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
-// ---- A/B switches of one-off experiments (all off by default) ----
-#ifndef FMM_AB_L64_VECTOR
-#define FMM_AB_L64_VECTOR 0      // 1: whole-wave rows take column ids through ds_bpermute into vector registers
-#endif
-#ifndef FMM_AB_Z_PLAIN_STORE
-#define FMM_AB_Z_PLAIN_STORE 0   // 1: finished Z rows are stored with plain (write-back) stores
-#endif
-#ifndef FMM_AB_EARLY_ROWS
-#define FMM_AB_EARLY_ROWS 0      // n > 0: one wave in n skips the segment phase and starts on rows at once
-#endif
-
 namespace fmm {
 
 // The library is compiled once per value type, as the reference is (-DDREAL).
@@ -761,7 +750,7 @@ __device__ __forceinline__ void load_chunk(EdgeChunk<IdxT> &c, const Params<IdxT
 template <int L>
 __device__ __forceinline__ int32_t chunk_entry(int32_t v, int e)
 {
-   if (L == 64 && !FMM_AB_L64_VECTOR) return __builtin_amdgcn_readlane(v, e);
+   if (L == 64) return __builtin_amdgcn_readlane(v, e);
    return __builtin_amdgcn_ds_bpermute(e << 2, v);
 }
 template <int L>
@@ -1323,17 +1312,8 @@ __device__ __forceinline__ void segments_phase(const Params<IdxT> &p, lds_table_
 
    const int lane = threadIdx.x & 63;
    const int sub = lane / L, sl = lane % L;
-#if FMM_AB_EARLY_ROWS > 0
-   const int64_t w_all = (int64_t)blockIdx.x * kWavesPerBlock + (threadIdx.x >> 6);
-   const int64_t n_all = (int64_t)gridDim.x * kWavesPerBlock;
-   constexpr int64_t kN = FMM_AB_EARLY_ROWS;
-   if (n_all >= 2 * kN && w_all % kN == kN - 1) return;                    // this wave starts on rows at once
-   const int64_t wave0 = n_all >= 2 * kN ? (kN - 1) * (w_all / kN) + w_all % kN : w_all;
-   const int64_t nwaves = n_all >= 2 * kN ? (n_all / kN) * (kN - 1) + ((n_all % kN) < (kN - 1) ? (n_all % kN) : (kN - 1)) : n_all;
-#else
    const int64_t wave0 = (int64_t)blockIdx.x * kWavesPerBlock + (threadIdx.x >> 6);
    const int64_t nwaves = (int64_t)gridDim.x * kWavesPerBlock;
-#endif
    const bool reads_x = op_reads_x<OP>(p.imessage);
    const int aop = p.imessage & 0xF0000;
 
@@ -1566,7 +1546,7 @@ __device__ __forceinline__ void rows_phase(const Params<IdxT> &p, lds_table_t ta
             load_slice<V, L, R, EXACT>(zin, zrow, sl, p.k);
             map2(acc, zin, acc, [](real_t a, real_t b) { return a + b; });
          }
-         store_slice<V, L, R, EXACT, !FMM_AB_Z_PLAIN_STORE>(zrow, acc, sl, p.k);
+         store_slice<V, L, R, EXACT, true>(zrow, acc, sl, p.k);
       }
    }
    chunk = nc > 0 ? resolve_claim<IdxT>(p, claimed, cur, nc, nchunks, lane) : -1;
