@@ -35,7 +35,8 @@ TRAFFIC_IS = ("L2-miss (fabric) bytes per call: FETCH_SIZE + WRITE_SIZE scaled b
 # the second configuration with a bandwidth target (gcn K=256), then the skewed ones.
 ALSO_DEFAULT = ("c3g", "c3", "c4", "c5")   # c3g and c3 share a graph
 PROFILE_OF = {"c2": "fused_kernel_sigmoid_k128_c2.md", "c3": "spmm_k256_c3_rmat22.md",
-              "c3g": "gcn_k256_c3g_rmat22.md", "c4": "tdist_k64_c4_rmat24.md", "c5": "sigmoid_k512_c5_zipf.md"}
+              "c3g": "gcn_k256_c3g_rmat22.md", "c4": "tdist_k64_c4_rmat24.md", "c5": "sigmoid_k512_c5_zipf.md",
+              "k32er": "tdist_k32_k32er.md", "k64er": "tdist_k64_k64er.md"}
 
 
 def measured_traffic_bytes(workload):
@@ -65,6 +66,9 @@ WORKLOADS = {
 for _k in range(32, 257, 32):
     WORKLOADS["k%der" % _k] = ("tdist K=%d, ER n=2^23 nnz=2^27 (%d-byte rows, Y of %g GiB)" % (_k, 4 * _k, _k / 32.0),
                                "t", _k, "tdist")
+    # the same graph and embeddings under the gcn tuple (gathers and adds only) and the sigmoid tuple
+    WORKLOADS["g%der" % _k] = ("gcn K=%d on the k%der graph" % (_k, _k), "g", _k, None)
+    WORKLOADS["s%der" % _k] = ("sigmoid K=%d on the k%der graph" % (_k, _k), "s", _k, "sigmoid")
 # What a row length costs: sigmoid K=512 over a Y of 2^21 rows (c5's), every row with the
 # same number of uniformly random neighbours, min(2^21, 2^25 / degree) rows.
 for _d in (1, 4, 16, 64, 512):
@@ -98,11 +102,12 @@ def make_workload(name, scale_down=0):
         n = (1 << 21) >> sd
         g = synth.zipf_graph(n, 1.8, min(1000000, n // 2), 40000000 >> sd, 5)
         return g, synth.uniform_matrix(n, 512, -0.5, 0.5, 5, 1), synth.uniform_matrix(n, 512, -0.5, 0.5, 5, 2)
-    if name.startswith("k") and name.endswith("er"):
+    if name[0] in "kgs" and name.endswith("er") and name[1:-2].isdigit():
         n = (1 << 23) >> sd
         k = int(name[1:-2])
         g = synth.er_graph(n, 8 * n, 7)
-        return g, synth.uniform_matrix(n, k, -1.0, 1.0, 7, 1), synth.uniform_matrix(n, k, -1.0, 1.0, 7, 2)
+        lim = 1.0 if name[0] != "s" else 2.0 / np.sqrt(k)          # sigmoid: keep the dots inside the table's range
+        return g, synth.uniform_matrix(n, k, -lim, lim, 7, 1), synth.uniform_matrix(n, k, -lim, lim, 7, 2)
     if name.startswith("u512d"):
         d = int(name[5:])
         n = (1 << 21) >> sd
@@ -309,6 +314,8 @@ _graphs = {}
 def workload_data(name):
     """make_workload(), the graph shared by workloads that differ in the op tuple only (c3/c3g, c4/c4g)."""
     key = {"c3g": "c3", "c4g": "c4"}.get(name, name)
+    if name[0] == "g" and name.endswith("er"):
+        key = "k" + name[1:]
     if key not in _graphs:
         _graphs.clear()                     # one graph at a time: the large ones take several GB of host memory
         _graphs[key] = cached_workload(key)

@@ -10,7 +10,7 @@ TKERN_MSG = {"g": fa.MSG_GCN, "m": fa.MSG_SPMM, "s": fa.MSG_SIGMOID, "t": fa.MSG
 
 def layout_for(k, vec_ok=True):
     """(V, L, S): floats per load, lanes per neighbour row, sub-waves per wave --
-    the rule in fusedmm_capi.hip:pick_shape."""
+    the rule of pick_shape in fusedmm_dispatch.hip."""
     if vec_ok and k % 4 == 0:
         if k <= 32:
             L = 8
