@@ -30,8 +30,10 @@ int launch_instance(const Params<idx_t> &p, const Launch &l)
    // Four workgroups (16 waves) per CU at most: with 8-16 gathers in flight per wave
    // that saturates the memory system, and more waves only evict each other's lines
    // (measured on the sigmoid K=128 benchmark: 1.307 ms at 4 per CU, 1.314 at 5, 1.335 at 6).
+   // (FUSEDMM_BLOCKS_PER_CU is capped at what stays resident: segments are dealt to the grid's waves by number, so a
+   // workgroup that has to wait for a free slot would hold its segments back until then)
    const int resident = occ < 4 ? occ : 4;
-   int64_t gr = (int64_t)l.num_cu * (l.blocks_per_cu > 0 ? l.blocks_per_cu : resident);
+   int64_t gr = (int64_t)l.num_cu * (l.blocks_per_cu > 0 ? (l.blocks_per_cu < occ ? l.blocks_per_cu : occ) : resident);
    if (gr > need) gr = need;
    if (gr < 1) gr = 1;
    Params<idx_t> pr = p;
