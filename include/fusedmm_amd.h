@@ -228,13 +228,13 @@ void fusedMM_amd_set_split(int64_t heavy_deg, int seg_len);
  * the environment variable FUSEDMM_SPLIT=heavy_deg,seg_len gave. */
 void fusedMM_amd_get_split(int64_t *heavy_deg, int *seg_len);
 
-/* Short rows one per group of lanes.  For K <= 64 a wavefront holds 4 (K > 32) or 8 neighbour rows at a
- * time; a group of that many consecutive CSR rows whose longest has no more than 8 edges per non-empty row
- * of the group (and at most 32 / 64 edges) is processed with one row per group of lanes, every row's edges
- * in order, instead of one row after the other across the whole wavefront.  1 (default; also
- * FUSEDMM_PACK_ROWS=on|auto) enables it, 0 (FUSEDMM_PACK_ROWS=off) disables it.  Which rows are taken that
- * way depends on the row pointers only; it changes the order in which such a row's edges are summed (same
- * values to rounding) and nothing else.  Returns the previous setting. */
+/* Short rows one per group of lanes.  For K <= 64 a wavefront holds S = 8 (K <= 32) or 4 neighbour rows at a time and
+ * keeps U = 8 gathers (4 in double precision) in flight for each.  A group of S consecutive CSR rows (row numbers
+ * g*S .. g*S+S-1) whose longest row has md <= S*U edges and ceil(md / U) <= (rows of the group that have edges) is
+ * processed with one row per group of lanes, every row's edges in order, instead of one row after the other across
+ * the whole wavefront.  1 (default; also FUSEDMM_PACK_ROWS=on|auto) enables it, 0 (FUSEDMM_PACK_ROWS=off) disables
+ * it.  Which rows are taken that way depends on the row pointers only; it changes the order in which such a row's
+ * edges are summed (same values to rounding) and nothing else.  Returns the previous setting. */
 int fusedMM_amd_set_pack_rows(int enable);
 
 /*

@@ -128,3 +128,83 @@ def test_random_general_tuple(seed):
     eps = float(np.finfo(np_v).eps)
     tol = 256 * eps * 200 * (float(np.abs(want).max()) + 1.0)
     assert float(np.abs(Z.astype(np.float64) - want.astype(np.float64)).max()) <= tol
+
+
+def _random_degrees(rng, rows):
+    """Row lengths of several characters in one matrix: stretches of Poisson lengths, stretches of empty rows,
+    power-law lengths, a few long rows."""
+    deg = np.zeros(rows, np.int64)
+    i = 0
+    while i < rows:
+        n = int(rng.integers(1, 40))
+        kind = int(rng.integers(0, 5))
+        if kind == 0:
+            d = rng.poisson(float(rng.choice([2, 8, 16, 30])), n)
+        elif kind == 1:
+            d = np.zeros(n, np.int64)
+        elif kind == 2:
+            d = np.minimum(rng.zipf(1.7, n), 300)
+        elif kind == 3:
+            d = rng.integers(0, 70, n)
+        else:
+            d = np.full(n, int(rng.choice([1, 8, 9, 16, 32, 33, 64, 65])))
+        deg[i:i + n] = d[:rows - i]
+        i += n
+    for _ in range(int(rng.integers(0, 3))):
+        deg[int(rng.integers(0, rows))] = int(rng.choice([150, 700, 3000]))
+    return deg
+
+
+@pytest.mark.parametrize("seed", range(_N or 40))
+def test_random_structure_matches_the_mirror_bit_for_bit(seed):
+    """Random mixtures of row lengths (which decide what is walked one row per sub-wave, what by the whole wavefront
+    and what in segments), widths, strides, thresholds and tuples: the library against the CPU mirror of its
+    order of operations, bit for bit."""
+    from fusedmm_amd import synth
+    rng = np.random.default_rng(9000 + seed)
+    bits = int(rng.choice([32, 64]))
+    vbits = int(rng.choice([32, 32, 64]))
+    np_v, u = (np.float32, np.uint32) if vbits == 32 else (np.float64, np.uint64)
+    rows, cols = int(rng.integers(1, 700)), int(rng.integers(1, 400))
+    k = int(rng.choice([4, 8, 20, 32, 36, 48, 64, 100, 128, 256, 260, 512]))
+    tkern, kind = [("g", None), ("m", None), ("s", "sigmoid"), ("t", "tdist"), ("f", "fr")][seed % 5]
+    beta = float(rng.choice([0.0, 1.0]))
+    deg = _random_degrees(rng, rows)
+    rowptr = np.concatenate([[0], np.cumsum(deg)])
+    nnz = int(rowptr[-1])
+    g = synth.graph_from_rowptr(rows, cols, rowptr, rng.integers(0, cols, max(nnz, 1), dtype=np.int64)[:nnz] if nnz else np.zeros(0, np.int64), None, bits)
+    if nnz == 0:
+        g["indx"] = np.zeros(1, g["indx"].dtype)
+        g["val"] = np.zeros(1, np.float32)
+    else:
+        g["val"] = synth.edge_values(nnz, seed)
+        if rng.random() < 0.3:
+            g = graphs.split_pointers(g, seed)
+    pad = lambda: 4 * int(rng.choice([0, 0, 1, 2]))              # strides that keep the 16-byte layout
+    ldx, ldy, ldz = k + pad(), k + pad(), k + pad()
+    lo, hi = (-0.5, 0.5) if tkern in ("s", "g", "m") else (-1.0, 1.0)
+    X = graphs.features(rows, ldx, seed, lo, hi, 1).astype(np_v)
+    Y = graphs.features(cols, ldy, seed, lo, hi, 2).astype(np_v)
+    if tkern == "f":
+        Y = (Y + np_v(3.0)).astype(np_v)                          # FR: keep X and Y apart (1/s)
+    Z0 = graphs.features(rows, ldz, seed, -1, 1, 3).astype(np_v)
+    m = rows if rng.random() < 0.6 else int(rng.integers(0, rows + 1))
+    sk = SOP_NAMES[kind] if kind else 0
+    split = gpu_api.default_split(k, vbits) if rng.random() < 0.4 else (int(rng.integers(20, 200)), int(rng.integers(8, 64)))
+    pack = bool(rng.random() < 0.8)
+    print("case", seed, dict(bits=bits, vbits=vbits, rows=rows, cols=cols, k=k, op=tkern, beta=beta, ld=(ldx, ldy, ldz), m=m,
+                             split=split, pack=pack, nnz=nnz), flush=True)
+    lib = fa.load(bits, vbits)
+    gpu_api.set_kind(sk, bits, vbits)
+    gpu_api.set_split(split[0], split[1], bits, vbits)
+    prev = lib.fusedMM_amd_set_pack_rows(1 if pack else 0)
+    try:
+        rc, Z = gpu_api.run(MSG[tkern], g, X, Y, Z0, beta=beta, bits=bits, m=m, k=k, ldx=ldx, ldy=ldy, ldz=ldz, vbits=vbits)
+    finally:
+        gpu_api.set_split(0, 0, bits, vbits)
+        lib.fusedMM_amd_set_pack_rows(prev)
+    assert rc == 0
+    want = gpu_api.oracle_mirror(orc(vbits), tkern, g, X, Y, Z0, beta, sk, k, split[0], split[1], m=m, pack=pack)
+    np.testing.assert_array_equal(Z.view(u), want.view(u))
+    np.testing.assert_array_equal(Z[m:], Z0[m:])
+    np.testing.assert_array_equal(Z[:, k:], Z0[:, k:])
