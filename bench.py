@@ -36,7 +36,8 @@ TRAFFIC_IS = ("L2-miss (fabric) bytes per call: FETCH_SIZE + WRITE_SIZE scaled b
 ALSO_DEFAULT = ("c3g", "c3", "c4", "c5")   # c3g and c3 share a graph
 PROFILE_OF = {"c2": "fused_kernel_sigmoid_k128_c2.md", "c3": "spmm_k256_c3_rmat22.md",
               "c3g": "gcn_k256_c3g_rmat22.md", "c4": "tdist_k64_c4_rmat24.md", "c5": "sigmoid_k512_c5_zipf.md",
-              "k32er": "tdist_k32_k32er.md", "k64er": "tdist_k64_k64er.md"}
+              "k32er": "tdist_k32_k32er.md", "k64er": "tdist_k64_k64er.md", "k128er": "tdist_k128_k128er.md",
+              "k256er": "tdist_k256_k256er.md"}
 
 
 def measured_traffic_bytes(workload):
@@ -259,8 +260,15 @@ def parse_args(argv=None):
     return ap.parse_args(argv)
 
 
+# Launch shapes of the gather probe: (workgroups per CU, gathers in flight per wavefront).  4 x 8 is the shape of
+# the fused kernel itself; 8 x 4, twice the waves each with half the queue, is the best of a sweep over 2-16 x 4-16 at
+# every row size from 128 bytes to 1 KiB.  The yardstick is the better of the two.
+GATHER_PROBE_SHAPES = ((4, 8), (8, 4))
+
+
 def run_gather_probe(torch, probes, n, row_bytes, stream):
-    """Read-only gather of 4 GiB of uniformly random rows of row_bytes out of a buffer of n rows."""
+    """Read-only gather of 4 GiB of uniformly random rows of row_bytes out of a buffer of n rows: the best rate over
+    GATHER_PROBE_SHAPES for plain and for non-temporal loads, and every shape's own figures under "shapes"."""
     dev = torch.device("cuda:0")
     nbytes = n * row_bytes
     src = torch.empty(nbytes // 4, dtype=torch.float32, device=dev).uniform_(-1, 1)
@@ -269,20 +277,23 @@ def run_gather_probe(torch, probes, n, row_bytes, stream):
     gen = torch.Generator(device=dev)
     gen.manual_seed(11)
     ids = torch.randint(0, n, (n_ids,), device=dev, dtype=torch.int64, generator=gen).to(torch.int32)
-    out = {"row_bytes": row_bytes, "buffer_bytes": nbytes, "gathered_bytes": n_ids * row_bytes}
-    for label, nt in (("plain_loads", 0), ("nontemporal_loads", 1)):
-        launch = lambda: probes.fusedMM_amd_gather_probe(src.data_ptr(), row_bytes, ids.data_ptr(), n_ids, 4, 8, nt,
-                                                         sink.data_ptr(), stream)
-        for _ in range(2):
-            assert launch() == 0
-        torch.cuda.synchronize()
-        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-        e0.record()
-        for _ in range(10):
-            launch()
-        e1.record()
-        torch.cuda.synchronize()
-        out[label + "_GBps"] = n_ids * row_bytes / (e0.elapsed_time(e1) / 10 * 1e-3) / 1e9
+    out = {"row_bytes": row_bytes, "buffer_bytes": nbytes, "gathered_bytes": n_ids * row_bytes, "shapes": {}}
+    for per_cu, in_flight in GATHER_PROBE_SHAPES:
+        shape = out["shapes"].setdefault("%dx%d" % (per_cu, in_flight), {})
+        for label, nt in (("plain_loads", 0), ("nontemporal_loads", 1)):
+            launch = lambda: probes.fusedMM_amd_gather_probe(src.data_ptr(), row_bytes, ids.data_ptr(), n_ids, per_cu,
+                                                             in_flight, nt, sink.data_ptr(), stream)
+            for _ in range(2):
+                assert launch() == 0
+            torch.cuda.synchronize()
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record()
+            for _ in range(10):
+                launch()
+            e1.record()
+            torch.cuda.synchronize()
+            shape[label + "_GBps"] = n_ids * row_bytes / (e0.elapsed_time(e1) / 10 * 1e-3) / 1e9
+            out[label + "_GBps"] = max(out.get(label + "_GBps", 0.0), shape[label + "_GBps"])
     del src, sink, ids
     return out
 
@@ -523,7 +534,11 @@ def measure(torch, fa, probes, name, steps, warmup, args, gather_probe, read_pro
         "value": value, "unit": "GFLOP/s", "steps": steps, "warmup": warmup, "ms_per_step": ms_per_step,
         "config": {"workload": "%s: %s" % (name, desc), "op": tkern, "K": k, "rows": m, "nnz": nnz,
                    "index_bits": bits, "beta": 0.0, "graph_gen_s": round(t_gen, 2),
-                   "pipeline": "general" if args.general else "optimised", "ldz": ldz},
+                   "pipeline": "general" if args.general else "optimised", "ldz": ldz,
+                   # when finished Z rows are written (fusedMM_amd_set_store_tick): "auto" holds them for a common
+                   # 82 us clock tick where Y is 1 GiB or more, and writes them as they finish otherwise
+                   "store_tick": os.environ.get("FUSEDMM_STORE_TICK", "auto"),
+                   "y_bytes": int(Y.shape[0]) * int(Y.shape[1]) * int(Y.itemsize)},
         "edges_per_s": nnz / (ms_per_step * 1e-3),
         "hbm_GBps_algorithmic": b_alg / (ms_per_step * 1e-3) / 1e9,
         "pct_peak_hbm": 100.0 * b_alg / (ms_per_step * 1e-3) / 1e9 / PEAK_HBM_GBPS,
@@ -552,7 +567,8 @@ def compact(name, r):
                          "frac": rl["frac"], "traffic": rl["traffic"], "traffic_from": rl["traffic_from"],
                          "frac_of_gather_probe": rl.get("frac_of_gather_probe"),
                          "gather_probe_GBps": (rl.get("gather_probe") or {}).get("plain_loads_GBps")},
-            "split": r["split"], "row_order_scattered": r["row_order"]["scattered"],
+            "split": r["split"], "row_order_scattered": r["row_order"]["scattered"], "store_tick": r["config"]["store_tick"],
+            "y_bytes": r["config"]["y_bytes"],
             "graph_gen_s": r["config"]["graph_gen_s"], "spot_check_vs_oracle": r["spot_check_vs_oracle"]}
 
 

@@ -38,7 +38,7 @@ EXPORTS = ("fusedMM_csr", "fusedMM_csr_stream", "fusedMM_csr_stream_noalloc", "f
            "fusedMM_amd_value_bytes", "fusedMM_amd_set_sop_kind", "fusedMM_amd_get_sop_kind",
            "fusedMM_amd_set_sop_callback", "fusedMM_amd_set_stage_callbacks", "fusedMM_amd_set_opt",
            "fusedMM_amd_set_validate", "fusedMM_amd_set_cache", "fusedMM_amd_invalidate",
-           "fusedMM_amd_last_host_phases", "fusedMM_amd_set_split", "fusedMM_amd_get_split", "fusedMM_amd_set_pack_rows", "fusedMM_amd_timing",
+           "fusedMM_amd_last_host_phases", "fusedMM_amd_set_split", "fusedMM_amd_get_split", "fusedMM_amd_set_pack_rows", "fusedMM_amd_set_store_tick", "fusedMM_amd_timing",
            "fusedMM_amd_timing_summary", "fusedMM_amd_timing_call", "fusedMM_amd_last_split",
            "fusedMM_amd_last_row_order", "fusedMM_amd_finalize")
 # the measuring aids of libfusedmm_amd_probes.so (csrc/fusedmm_probes.h): not part of the product's ABI
@@ -102,6 +102,8 @@ def load(index_bits=32, value_bits=32):
     lib.fusedMM_amd_get_split.restype = None
     lib.fusedMM_amd_set_pack_rows.argtypes = [C.c_int]
     lib.fusedMM_amd_set_pack_rows.restype = C.c_int
+    lib.fusedMM_amd_set_store_tick.argtypes = [C.c_int]
+    lib.fusedMM_amd_set_store_tick.restype = C.c_int
     lib.fusedMM_amd_last_row_order.argtypes = [vp, vp, vp]
     lib.fusedMM_amd_last_row_order.restype = C.c_int
     lib.fusedMM_amd_set_stage_callbacks.argtypes = [vp, vp, vp, vp]

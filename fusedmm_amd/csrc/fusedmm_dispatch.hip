@@ -148,6 +148,13 @@ int run_slab(const Args &a, const Plan &pl, int sop_kind, hipStream_t stream, in
    p.imessage = a.imessage;
    p.row_order = g.row_order;
    p.pack_rows = (g.pack != 1 && sh.V == 4 && sh.L <= 16) ? 1 : 0;
+   // Finished rows of Z wait in LDS for a common store tick (82 us) where the gathered matrix is several times the
+   // 256 MiB last-level cache, 1 GiB and more: there the gathers run at the memory's own rate and a thin stream of
+   // stores between them costs several times its share (2^23 rows of 16 edges, K = 64 ... 256: 9-14 % of the call).
+   // Where much of Y is served from that cache the stores are not what limits, and the bookkeeping costs half a
+   // per cent (sigmoid K=128 on 2^20 nodes, Y of 512 MiB).
+   if (g.store_shift >= 0) p.store_shift = g.store_shift;
+   else p.store_shift = (a.n * a.ldy * (int64_t)kValBytes >= (1ll << 30)) ? 13 : 0;
 
    // heavy-row split: segments of about 1 MiB of gathered rows but at most 2048 edges
    // (measured best on the R-MAT and power-law benchmark graphs: shorter segments pay

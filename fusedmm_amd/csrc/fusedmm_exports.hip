@@ -385,6 +385,15 @@ int fusedMM_amd_set_pack_rows(int mode)
    return prev;
 }
 
+int fusedMM_amd_set_store_tick(int shift)
+{
+   std::lock_guard<std::mutex> lock(g.mu);
+   read_env_once();
+   const int prev = g.store_shift;
+   g.store_shift = shift == 0 ? 0 : ((shift >= 8 && shift <= 24) ? shift : -1);
+   return prev;
+}
+
 void fusedMM_amd_timing(int enable)
 {
    std::lock_guard<std::mutex> lock(g.mu);

@@ -118,6 +118,7 @@ struct Globals {
    int validate = 0;
    int row_order = 0;         // 0 auto, 1 first to last, 2 scattered stretches (FUSEDMM_ROW_ORDER)
    int pack = 0;              // short rows one per sub-wave: 0 auto, 1 never, 2 always where the shape allows (FUSEDMM_PACK_ROWS)
+   int store_shift = -1;      // finished Z rows leave together when the 100 MHz clock >> this changes: -1 auto, 0 never (FUSEDMM_STORE_TICK)
    int cache = 0;             // 1: keep device mirrors of read-only host operands between calls
    unsigned long long cache_clock = 0;
    double phase_ms[3] = {0, 0, 0};   // upload, kernels, download of the last host-pointer call

@@ -126,6 +126,8 @@ struct Params {
    int row_counters;       // claim counters in use: kRowCounters; 1 when the grid has fewer waves; 0: wave w takes chunk w
    int row_order;          // 0: decided from the classify kernel's sample; 1: first to last; 2: scattered stretches
    int pack_rows;          // 1: groups of short rows are walked one row per sub-wave (sub-waves of 8 or 16 lanes)
+   int store_shift;        // finished Z rows leave LDS when the 100 MHz clock >> store_shift changes; 0: stored as they finish
+   int stage_vecs;         // LDS each wavefront has for such rows, in 4-element registers (the launch's dynamic LDS / waves)
 };
 
 // ---- wave primitives --------------------------------------------------------
@@ -890,6 +892,163 @@ __device__ __forceinline__ lds_table_t stage_table(const real_t *gtab, real_t *l
    return (lds_table_t)lds;      // read only when `need` held
 }
 
+// ---- finished Z rows leave together -----------------------------------------------
+// A finished row of Z is one store of 128 bytes to a few KiB, and on rows of a few dozen
+// edges such stores are a twentieth of the bytes a call moves.  Sent out one by one as
+// rows finish they reach the memory system as a thin, steady trickle between random
+// reads, and cost it several times their share (a 16-edge graph at K=512: 4 GB of Z took
+// as long as 23 GB of gathers).  So finished rows wait in LDS, and every wavefront of
+// the grid sends its waiting rows when the same clock tick passes: the device's constant
+// 100 MHz counter (s_memrealtime, one counter for all compute dies) shifted right by
+// store_shift.  The stores of the whole grid then arrive in bursts a few microseconds
+// long, once per period, with nothing but reads in between; what is summed, and in which
+// order, does not change.  A wavefront whose LDS share fills up before the tick sends
+// early.  Each wavefront has its share of the workgroup's dynamic LDS, in slots of one sub-wave row (L lanes x
+// R registers) followed by the slots' destinations.  Rows to be cleared (empty rows under the
+// overwrite rule) need no slot, only their address.
+constexpr int kClearList = 32;          // rows waiting to be cleared, per wavefront
+struct RowStage {
+   real4 *slots;        // this wavefront's share of the workgroup's staging area: cap slots, ...
+   real_t **to;         // ... then where each slot goes (nullptr: nowhere), ...
+   real_t **clear;      // ... then the rows waiting to be cleared
+   int cap;             // slots this wavefront has
+   int n, nclear;       // slots in use, rows to clear
+   unsigned int tick;   // clock >> shift at the last look
+   int shift;           // 0: rows are stored as they finish
+};                      // (every member is wave-uniform)
+
+// The staging area is the workgroup's dynamic LDS: stage_vecs registers' worth (real4) per wavefront, sized by
+// the host to what the CU's LDS leaves each resident workgroup.
+template <int L, int R, typename IdxT>
+__device__ __forceinline__ void stage_begin(RowStage &st, const Params<IdxT> &p, real4 *lds)
+{
+   constexpr int S = 64 / L;
+   constexpr int kSlotBytes = L * R * (int)sizeof(real4);
+   const int wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
+   const int share = p.stage_vecs * (int)sizeof(real4);
+   int cap = (share - kClearList * (int)sizeof(real_t *)) / (kSlotBytes + (int)sizeof(real_t *));
+   cap = cap > 64 ? 64 : (cap < 0 ? 0 : cap);
+   st.slots = lds + wave * p.stage_vecs;
+   st.to = reinterpret_cast<real_t **>(st.slots + cap * L * R);
+   st.clear = st.to + cap;
+   st.cap = cap;
+   st.n = 0;
+   st.nclear = 0;
+   st.shift = cap >= 2 * S ? p.store_shift : 0;     // room for two rows, or two packed groups, at least
+   st.tick = st.shift ? (unsigned int)(__builtin_amdgcn_s_memrealtime() >> st.shift) : 0u;
+}
+
+template <int V, int L, int R, bool EXACT>
+__device__ __forceinline__ void stage_flush(RowStage &st, int lane, int k)
+{
+   constexpr int S = 64 / L;
+   const int sub = (L == 64) ? 0 : lane / L, sl = (L == 64) ? lane : lane % L;
+   __builtin_amdgcn_wave_barrier();
+   for (int i = 0; i < st.n; i += S)
+   {
+      const int slot = i + sub;
+      if (slot < st.n)
+      {
+         real_t *to = st.to[slot];
+         if (to)
+         {
+            Slice<R> row;
+#pragma unroll
+            for (int r = 0; r < R; r++) row.v[r] = st.slots[(slot * R + r) * L + sl];
+            store_slice<V, L, R, EXACT, true>(to, row, sl, k);
+         }
+      }
+   }
+   for (int i = 0; i < st.nclear; i += S)
+   {
+      const int at = i + sub;
+      if (at < st.nclear)
+      {
+         Slice<R> zero;
+#pragma unroll
+         for (int r = 0; r < R; r++) zero.v[r] = zero4();
+         store_slice<V, L, R, EXACT, true>(st.clear[at], zero, sl, k);
+      }
+   }
+   __builtin_amdgcn_wave_barrier();
+   st.n = 0;
+   st.nclear = 0;
+}
+
+// Has the tick passed?  Then everything waiting goes out.  `clock` is a reading of the 100 MHz counter taken a
+// little earlier (before the row was walked: the read is under way while the row is).
+template <int V, int L, int R, bool EXACT>
+__device__ __forceinline__ void stage_tick(RowStage &st, unsigned long long clock, int lane, int k)
+{
+   if (st.shift == 0) return;
+   const unsigned int now = (unsigned int)(clock >> st.shift);
+   if (now != st.tick)
+   {
+      if (st.n | st.nclear) stage_flush<V, L, R, EXACT>(st, lane, k);
+      st.tick = now;
+   }
+}
+
+// One finished row, held by the wavefront's first sub-wave; zrow is wave-uniform.
+template <int V, int L, int R, bool EXACT>
+__device__ __forceinline__ void stage_row(RowStage &st, real_t *zrow, const Slice<R> &acc, int lane, int k)
+{
+   const int sub = (L == 64) ? 0 : lane / L, sl = (L == 64) ? lane : lane % L;
+   if (st.shift == 0)
+   {
+      if (sub == 0) store_slice<V, L, R, EXACT, true>(zrow, acc, sl, k);
+      return;
+   }
+   if (st.n >= st.cap) stage_flush<V, L, R, EXACT>(st, lane, k);   // (a packed group may have filled the last slot)
+   if (sub == 0)
+   {
+#pragma unroll
+      for (int r = 0; r < R; r++) st.slots[(st.n * R + r) * L + sl] = acc.v[r];
+   }
+   if (lane == 0) st.to[st.n] = zrow;
+   st.n++;
+}
+
+// One row per sub-wave (a packed group): sub-wave s holds a row for `zrow` (its own; nullptr: nothing to store).
+template <int V, int L, int R, bool EXACT>
+__device__ __forceinline__ void stage_group(RowStage &st, real_t *zrow, const Slice<R> &acc, int lane, int k)
+{
+   constexpr int S = 64 / L;
+   const int sub = lane / L, sl = lane % L;
+   if (st.shift == 0)
+   {
+      if (zrow) store_slice<V, L, R, EXACT, true>(zrow, acc, sl, k);
+      return;
+   }
+   if (st.n + S > st.cap) stage_flush<V, L, R, EXACT>(st, lane, k);
+   const int slot = st.n + sub;
+#pragma unroll
+   for (int r = 0; r < R; r++) st.slots[(slot * R + r) * L + sl] = acc.v[r];
+   if (sl == 0) st.to[slot] = zrow;
+   st.n += S;
+}
+
+// An empty row under the overwrite rule: to be cleared; zrow is wave-uniform.
+template <int V, int L, int R, bool EXACT>
+__device__ __forceinline__ void stage_clear(RowStage &st, real_t *zrow, int lane, int k)
+{
+   const int sub = (L == 64) ? 0 : lane / L, sl = (L == 64) ? lane : lane % L;
+   if (st.shift == 0)
+   {
+      if (sub == 0)
+      {
+         Slice<R> zero;
+#pragma unroll
+         for (int r = 0; r < R; r++) zero.v[r] = zero4();
+         store_slice<V, L, R, EXACT, true>(zrow, zero, sl, k);
+      }
+      return;
+   }
+   if (st.nclear >= kClearList) stage_flush<V, L, R, EXACT>(st, lane, k);
+   if (lane == 0) st.clear[st.nclear] = zrow;
+   st.nclear++;
+}
+
 // ---- short rows, one per sub-wave --------------------------------------------------
 // A wavefront walks a row with all its S = 64/L sub-waves: S*U edges are gathered at a
 // time.  Rows much shorter than that leave most of those gathers unused (a 16-edge row
@@ -915,7 +1074,7 @@ __device__ __forceinline__ bool packs(int64_t md, int nz, int64_t heavy_deg)
 // longest row of the group.  All lanes of the wave call this together.
 template <int V, int L, int R, bool EXACT, int OP, int SOPK, int U, typename IdxT>
 __device__ __forceinline__ void packed_group(const Params<IdxT> &p, int64_t row_first, IdxT jb, IdxT je, int md, int lane,
-                                             lds_table_t tab)
+                                             lds_table_t tab, RowStage &st)
 {
    static_assert(L == 8 || L == 16, "sub-waves of 8 or 16 lanes");
    constexpr int P = 16 / L;                 // column ids a lane holds per fetch: 16 ids per sub-wave and fetch
@@ -1024,19 +1183,19 @@ __device__ __forceinline__ void packed_group(const Params<IdxT> &p, int64_t row_
       }
    }
 
+   bool stores;
    if (deg > 0)
    {
-      if (generic && aop == kAopNoop) return;             // no accumulate stage: Z is left alone
+      stores = !(generic && aop == kAopNoop);             // no accumulate stage: Z is left alone
       if (!generic && !p.beta_zero)
       {
          Slice<R> zin;
          load_slice<V, L, R, EXACT>(zin, zrow, sl, p.k);
          map2(acc, zin, acc, [](real_t a, real_t b) { return a + b; });
       }
-      store_slice<V, L, R, EXACT, true>(zrow, acc, sl, p.k);
    }
-   else if (!generic && p.beta_zero && row < p.m)
-      store_slice<V, L, R, EXACT, true>(zrow, acc, sl, p.k);   // empty row under the overwrite rule: zeros
+   else stores = !generic && p.beta_zero && row < p.m;    // empty row under the overwrite rule: zeros
+   stage_group<V, L, R, EXACT>(st, stores ? zrow : nullptr, acc, lane, p.k);
 }
 
 // Does the row phase take the stretches of 64 chunks in scattered order?  When rows are claimed dynamically,
@@ -1373,8 +1532,10 @@ __device__ __forceinline__ void segments_phase(const Params<IdxT> &p, lds_table_
 
 // ---- phase B of the fused kernel: one wavefront per row ---------------------------
 template <int V, int L, int R, bool EXACT, int OP, int SOPK, int U, typename IdxT>
-__device__ __forceinline__ void rows_phase(const Params<IdxT> &p, lds_table_t tab)
+__device__ __forceinline__ void rows_phase(const Params<IdxT> &p, lds_table_t tab, real4 *stage_lds)
 {
+   RowStage st;
+   stage_begin<L, R, IdxT>(st, p, stage_lds);
    const int lane = threadIdx.x & 63;
    const int sub = lane / L, sl = lane % L;
    const bool reads_x = op_reads_x<OP>(p.imessage);
@@ -1447,7 +1608,9 @@ __device__ __forceinline__ void rows_phase(const Params<IdxT> &p, lds_table_t ta
             {
                // sub-wave s takes row row0 + g0 + s: its pointers are in lane g0 + s
                const IdxT gb = chunk_entry<L>(my_b, g0 + lane / L), ge = chunk_entry<L>(my_e, g0 + lane / L);
-               packed_group<V, L, R, EXACT, OP, SOPK, U, IdxT>(p, row0 + g0, gb, ge > gb ? ge : gb, (int)md, lane, tab);
+               const unsigned long long clock = __builtin_amdgcn_s_memrealtime();
+               packed_group<V, L, R, EXACT, OP, SOPK, U, IdxT>(p, row0 + g0, gb, ge > gb ? ge : gb, (int)md, lane, tab, st);
+               stage_tick<V, L, R, EXACT>(st, clock, lane, p.k);
                packed_rows |= gmask;
             }
          }
@@ -1478,13 +1641,7 @@ __device__ __forceinline__ void rows_phase(const Params<IdxT> &p, lds_table_t ta
       {
          // empty row (about half the rows of an R-MAT graph): nothing to gather; the
          // overwrite rule still clears Z, every other rule leaves it alone
-         if (!generic && p.beta_zero && sub == 0)
-         {
-            Slice<R> zero;
-#pragma unroll
-            for (int r = 0; r < R; r++) zero.v[r] = zero4();
-            store_slice<V, L, R, EXACT, true>(zrow, zero, sl, p.k);
-         }
+         if (!generic && p.beta_zero) stage_clear<V, L, R, EXACT>(st, zrow, lane, p.k);
          continue;
       }
       if (generic && aop == kAopNoop) continue;   // general semantics with no accumulate stage: Z is left alone
@@ -1535,22 +1692,23 @@ __device__ __forceinline__ void rows_phase(const Params<IdxT> &p, lds_table_t ta
             for (int r = 0; r < R; r++) xs_next.v[r] = zero4();
          }
       }
+      const unsigned long long clock = __builtin_amdgcn_s_memrealtime();
       walk_edges<V, L, R, EXACT, OP, SOPK, U, IdxT>(acc, xs, p, jb, je, first, nb, ne, lane, tab);
       merge_subwaves<L, R, OP>(acc, p.imessage);
 
-      if (sub == 0)
+      if (sub == 0 && !generic && !p.beta_zero)
       {
-         if (!generic && !p.beta_zero)
-         {
-            Slice<R> zin;
-            load_slice<V, L, R, EXACT>(zin, zrow, sl, p.k);
-            map2(acc, zin, acc, [](real_t a, real_t b) { return a + b; });
-         }
-         store_slice<V, L, R, EXACT, true>(zrow, acc, sl, p.k);
+         Slice<R> zin;
+         load_slice<V, L, R, EXACT>(zin, zrow, sl, p.k);
+         map2(acc, zin, acc, [](real_t a, real_t b) { return a + b; });
       }
+      stage_row<V, L, R, EXACT>(st, zrow, acc, lane, p.k);
+      stage_tick<V, L, R, EXACT>(st, clock, lane, p.k);
    }
+   if (st.nclear) stage_tick<V, L, R, EXACT>(st, __builtin_amdgcn_s_memrealtime(), lane, p.k);   // a claim of empty rows
    chunk = nc > 0 ? resolve_claim<IdxT>(p, claimed, cur, nc, nchunks, lane) : -1;
    }
+   if (st.n | st.nclear) stage_flush<V, L, R, EXACT>(st, lane, p.k);
 }
 
 // Every wavefront ends here.  The last workgroup to finish, when nobody reads the
@@ -1607,14 +1765,23 @@ __device__ __forceinline__ void retire_wave(const Params<IdxT> &p)
 // rows (phase A), then claims ordinary rows until none are left (phase B).  One
 // kernel, so the short rows fill in behind the long segments instead of waiting
 // for them at a kernel boundary.
+extern __shared__ __attribute__((aligned(32))) unsigned char fmm_dynamic_lds[];
+
 template <int V, int L, int R, bool EXACT, int OP, int SOPK, int U, typename IdxT>
-__global__ __launch_bounds__(kBlockThreads) void fused_kernel(const Params<IdxT> p)
+// The float / int32 instances whose rows take one register per lane on sub-waves of 32 lanes or fewer are held to
+// 128 vector registers, four wavefronts per SIMD: they fit but for a few spilled values, and measured faster that
+// way than with the 130-145 registers the compiler takes when left alone (K=32 on 2^23 nodes: 3.18 against 3.42 ms;
+// K=64 on R-MAT 24: 23.1 against 23.7).  The wider instances and the other libraries keep the compiler's own
+// allocation: held to 128 registers, K=256 lost 2.5 %, and the int64 and double instances 4-6 % at K=64.
+#define FMM_MIN_WAVES ((R == 1 && L <= 32 && OP != OP_GENERIC && sizeof(IdxT) == 4 && sizeof(real_t) == 4) ? 4 : 1)
+__global__ __launch_bounds__(kBlockThreads, FMM_MIN_WAVES) void fused_kernel(const Params<IdxT> p)
 {
    __shared__ real_t lds_tab[(OP >= OP_DOT) ? kSigmoidTableSize : 1];
    const bool uses_sop = (OP == OP_DOT || OP == OP_DIST || (OP == OP_GENERIC && (p.imessage & 0xF00) == kSopUdef));
    const lds_table_t tab = stage_table(p.sigmoid_table, lds_tab, (OP >= OP_DOT) && uses_sop && (SOPK >= 0 ? SOPK : p.sop_kind) == SOP_SIGMOID);
    segments_phase<V, L, R, EXACT, OP, SOPK, U, IdxT>(p, tab);
-   rows_phase<V, L, R, EXACT, OP, SOPK, U, IdxT>(p, tab);
+   // finished Z rows wait in the dynamic LDS for the grid's common store tick
+   rows_phase<V, L, R, EXACT, OP, SOPK, U, IdxT>(p, tab, reinterpret_cast<real4 *>(fmm_dynamic_lds));
    retire_wave<IdxT>(p);
 }
 

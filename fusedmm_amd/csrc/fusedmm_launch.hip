@@ -17,12 +17,37 @@ int launch_instance(const Params<idx_t> &p, const Launch &l)
 {
    // persistent grid: as many blocks as stay resident; waves share out the
    // queued segments, then claim rows
-   static int occ = 0;
+   static int occ = 0, occ_staged = 0, stage_lds = 0;
    if (occ == 0)
    {
-      FMM_HIP(hipOccupancyMaxActiveBlocksPerMultiprocessor(&occ, fused_kernel<V, L, R, EXACT, OP, SOPK, U, idx_t>, kBlockThreads, 0));
+      const auto kernel = fused_kernel<V, L, R, EXACT, OP, SOPK, U, idx_t>;
+      FMM_HIP(hipOccupancyMaxActiveBlocksPerMultiprocessor(&occ, kernel, kBlockThreads, 0));
       if (occ < 1) occ = 1;
+      // Dynamic LDS for the rows that wait for the store tick: what a CU's 160 KiB leave each of the workgroups
+      // that are resident anyway (four at most) beside the kernel's own static LDS, within the 64 KiB one
+      // workgroup may have; then checked against the runtime's own count, and shrunk until residency is kept.
+      hipFuncAttributes attr;
+      FMM_HIP(hipFuncGetAttributes(&attr, reinterpret_cast<const void *>(kernel)));
+      const int want = occ < 4 ? occ : 4;
+      int lds = 163840 / want - (int)attr.sharedSizeBytes - 512;
+      if (lds > 65536 - (int)attr.sharedSizeBytes) lds = 65536 - (int)attr.sharedSizeBytes;
+      lds = lds > 0 ? lds / 1024 * 1024 : 0;
+      int got = occ;
+      while (lds > 0)
+      {
+         got = 0;
+         if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&got, kernel, kBlockThreads, (size_t)lds) == hipSuccess && got >= want) break;
+         (void)hipGetLastError();
+         lds -= 1024;
+      }
+      if (lds > 49152) (void)hipFuncSetAttribute(reinterpret_cast<const void *>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, lds);
+      (void)hipGetLastError();
+      stage_lds = lds > 0 ? lds : 0;
+      occ_staged = lds > 0 ? got : occ;
    }
+   const bool staged = p.store_shift > 0 && stage_lds > 0;
+   const int dyn_lds = staged ? stage_lds : 0;
+   const int occ_now = staged ? occ_staged : occ;
    // enough blocks for the rows, or for the segments the caller's nnz could give rise to
    int64_t need = (p.m + kWavesPerBlock - 1) / kWavesPerBlock;
    const int64_t need_segs = (l.nnz_hint / p.seg_len + kWavesPerBlock - 1) / kWavesPerBlock;
@@ -32,11 +57,13 @@ int launch_instance(const Params<idx_t> &p, const Launch &l)
    // (measured on the sigmoid K=128 benchmark: 1.307 ms at 4 per CU, 1.314 at 5, 1.335 at 6).
    // (FUSEDMM_BLOCKS_PER_CU is capped at what stays resident: segments are dealt to the grid's waves by number, so a
    // workgroup that has to wait for a free slot would hold its segments back until then)
-   const int resident = occ < 4 ? occ : 4;
-   int64_t gr = (int64_t)l.num_cu * (l.blocks_per_cu > 0 ? (l.blocks_per_cu < occ ? l.blocks_per_cu : occ) : resident);
+   const int resident = occ_now < 4 ? occ_now : 4;
+   int64_t gr = (int64_t)l.num_cu * (l.blocks_per_cu > 0 ? (l.blocks_per_cu < occ_now ? l.blocks_per_cu : occ_now) : resident);
    if (gr > need) gr = need;
    if (gr < 1) gr = 1;
    Params<idx_t> pr = p;
+   pr.stage_vecs = dyn_lds / (kWavesPerBlock * (int)sizeof(real4));
+   if (!staged) pr.store_shift = 0;
    const int64_t nchunks = (p.m + kRowsPerClaim - 1) / kRowsPerClaim;
    if (nchunks <= gr * kWavesPerBlock) pr.row_counters = 0;   // one chunk per wave at most: static
    else pr.row_counters = (gr * kWavesPerBlock >= kRowCounters) ? kRowCounters : 1;
@@ -45,7 +72,7 @@ int launch_instance(const Params<idx_t> &p, const Launch &l)
    if (l.ev) FMM_HIP(hipEventRecord(l.ev[0], l.stream));
    hipLaunchKernelGGL((classify_kernel<idx_t>), dim3((unsigned int)gc), dim3(kBlockThreads), 0, l.stream, p);
    if (l.ev) FMM_HIP(hipEventRecord(l.ev[1], l.stream));
-   hipLaunchKernelGGL((fused_kernel<V, L, R, EXACT, OP, SOPK, U, idx_t>), dim3((unsigned int)gr), dim3(kBlockThreads), 0, l.stream, pr);
+   hipLaunchKernelGGL((fused_kernel<V, L, R, EXACT, OP, SOPK, U, idx_t>), dim3((unsigned int)gr), dim3(kBlockThreads), (size_t)dyn_lds, l.stream, pr);
    if (l.ev) FMM_HIP(hipEventRecord(l.ev[2], l.stream));
    // one workgroup per heavy row and pass of 256 columns
    const unsigned int col_passes = (unsigned int)((p.k + kBlockThreads - 1) / kBlockThreads);

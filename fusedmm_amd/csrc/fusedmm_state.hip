@@ -50,6 +50,11 @@ void read_env_once()
       g.row_order = !strcmp(e, "plain") ? 1 : (!strcmp(e, "scattered") ? 2 : 0);
    if (const char *e = getenv("FUSEDMM_PACK_ROWS"))   // "auto", "off" or "on"
       g.pack = !strcmp(e, "off") ? 1 : (!strcmp(e, "on") ? 2 : 0);
+   if (const char *e = getenv("FUSEDMM_STORE_TICK"))   // "auto", "off" or the shift (8 ... 24)
+   {
+      const int v = atoi(e);
+      g.store_shift = !strcmp(e, "off") ? 0 : ((v >= 8 && v <= 24) ? v : -1);
+   }
    if (const char *e = getenv("FUSEDMM_SPLIT"))   // "heavy_deg,seg_len", as fusedMM_amd_set_split
    {
       long long h = 0;

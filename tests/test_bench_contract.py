@@ -83,7 +83,8 @@ def test_the_default_run_also_times_the_other_bandwidth_target_and_the_skewed_gr
     assert bench.ALSO_DEFAULT[0] == "c3g" and set(bench.ALSO_DEFAULT) == {"c3g", "c4", "c5", "c3"}
     assert all(w in bench.WORKLOADS and w in bench.PROFILE_OF for w in bench.ALSO_DEFAULT)
     full = {"value": 1.0, "unit": "GFLOP/s", "steps": 10, "warmup": 2, "ms_per_step": 2.0, "edges_per_s": 3.0,
-            "config": {"workload": "c3g: x", "op": "g", "K": 256, "rows": 4, "nnz": 5, "graph_gen_s": 1.0},
+            "config": {"workload": "c3g: x", "op": "g", "K": 256, "rows": 4, "nnz": 5, "graph_gen_s": 1.0, "store_tick": "auto",
+                       "y_bytes": 4096},
             "split": {"heavy_rows": 1, "segments": 2, "overflow": 0}, "row_order": {"scattered": True},
             "spot_check_vs_oracle": True,
             "roofline": {"bound": "hbm", "achieved": 6400.0, "peak": 8000.0, "unit": "GB/s", "frac": 0.8, "traffic": 7,
@@ -94,6 +95,8 @@ def test_the_default_run_also_times_the_other_bandwidth_target_and_the_skewed_gr
         assert key in c, key
     assert c["roofline"]["frac"] == 0.8 and c["roofline"]["traffic"] == 7 and c["roofline"]["frac_of_gather_probe"] == 1.1
     assert c["roofline"]["gather_probe_GBps"] == 5800.0 and c["kernel_ms"] == 1.9 and c["row_order_scattered"] is True
+    assert c["store_tick"] == "auto" and c["y_bytes"] == 4096
+    assert (4, 8) in bench.GATHER_PROBE_SHAPES and len(bench.GATHER_PROBE_SHAPES) >= 2     # the kernel's own launch shape and the probe's best
     # the narrow-row workloads: 2^23 rows of 128 and 256 bytes, 2^27 edges
     g, X, Y = bench.make_workload("k32er", 10)
     assert g["rows"] == 8192 and g["nnz"] == 16 * 8192 and X.shape == (8192, 32) and X is not Y
