@@ -153,8 +153,12 @@ int run_slab(const Args &a, const Plan &pl, int sop_kind, hipStream_t stream, in
    // stores between them costs several times its share (2^23 rows of 16 edges, K = 64 ... 256: 9-14 % of the call).
    // Where much of Y is served from that cache the stores are not what limits, and the bookkeeping costs half a
    // per cent (sigmoid K=128 on 2^20 nodes, Y of 512 MiB).
+   // The period is the longest one a wavefront's share of LDS still covers: 82 us, or 41 us where rows average
+   // fewer than 10 edges and the shares fill twice as fast (2^21 rows of 4 edges at K=512: 4.43 ms at 41 us, 4.57 at
+   // 82, 4.77 with rows written as they finish; rows of 16 edges: 13.8, 12.7, 14.6).
    if (g.store_shift >= 0) p.store_shift = g.store_shift;
-   else p.store_shift = (a.n * a.ldy * (int64_t)kValBytes >= (1ll << 30)) ? 13 : 0;
+   else if (a.n * a.ldy * (int64_t)kValBytes < (1ll << 30)) p.store_shift = 0;
+   else p.store_shift = (a.m > 0 && a.nnz / a.m < 10) ? 12 : 13;
 
    // heavy-row split: segments of about 1 MiB of gathered rows but at most 2048 edges
    // (measured best on the R-MAT and power-law benchmark graphs: shorter segments pay

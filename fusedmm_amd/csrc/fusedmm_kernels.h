@@ -907,55 +907,85 @@ __device__ __forceinline__ lds_table_t stage_table(const real_t *gtab, real_t *l
 // R registers) followed by the slots' destinations.  Rows to be cleared (empty rows under the
 // overwrite rule) need no slot, only their address.
 constexpr int kClearList = 32;          // rows waiting to be cleared, per wavefront
+
+// What a wavefront carries from row to row is four scalars; where its slots and lists lie is worked out from the
+// kernel's arguments when a row is put down or the rows go out (scalar registers are the scarce kind in this kernel).
 struct RowStage {
-   real4 *slots;        // this wavefront's share of the workgroup's staging area: cap slots, ...
-   real_t **to;         // ... then where each slot goes (nullptr: nowhere), ...
-   real_t **clear;      // ... then the rows waiting to be cleared
-   int cap;             // slots this wavefront has
+   int cap;             // slots this wavefront has; 0: rows are stored as they finish
    int n, nclear;       // slots in use, rows to clear
-   unsigned int tick;   // clock >> shift at the last look
-   int shift;           // 0: rows are stored as they finish
+   unsigned int tick;   // clock >> store_shift at the last look
 };                      // (every member is wave-uniform)
+
+extern __shared__ __attribute__((aligned(32))) unsigned char fmm_dynamic_lds[];
+
+// Registers (real4) per slot: L*R, or only those that hold elements of the row when K is not a multiple of 4*L
+// (16-byte layout: register r of lane sl is element-vector r*L + sl; vectors past the row's end hold nothing).
+template <int V, int L, int R, bool EXACT, typename IdxT>
+__device__ __forceinline__ int stage_width(const Params<IdxT> &p)
+{
+   return (V == 4 && !EXACT) ? (p.k + 3) / 4 : L * R;
+}
+// This wavefront's share of the staging area: cap slots, then where each slot goes (nullptr: nowhere), then the
+// rows waiting to be cleared.
+template <typename IdxT>
+__device__ __forceinline__ real4 *stage_slots(const Params<IdxT> &p)
+{
+   const int wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
+   return reinterpret_cast<real4 *>(fmm_dynamic_lds) + wave * p.stage_vecs;
+}
+template <int V, int L, int R, bool EXACT, typename IdxT>
+__device__ __forceinline__ real_t **stage_to(const Params<IdxT> &p, const RowStage &st)
+{
+   return reinterpret_cast<real_t **>(stage_slots<IdxT>(p) + st.cap * stage_width<V, L, R, EXACT, IdxT>(p));
+}
 
 // The staging area is the workgroup's dynamic LDS: stage_vecs registers' worth (real4) per wavefront, sized by
 // the host to what the CU's LDS leaves each resident workgroup.
-template <int L, int R, typename IdxT>
-__device__ __forceinline__ void stage_begin(RowStage &st, const Params<IdxT> &p, real4 *lds)
+template <int V, int L, int R, bool EXACT, bool STAGED, typename IdxT>
+__device__ __forceinline__ void stage_begin(RowStage &st, const Params<IdxT> &p)
 {
    constexpr int S = 64 / L;
-   constexpr int kSlotBytes = L * R * (int)sizeof(real4);
-   const int wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
+   if constexpr (!STAGED)
+   {
+      st.cap = 0;
+      st.n = 0;
+      st.nclear = 0;
+      st.tick = 0u;
+      return;
+   }
    const int share = p.stage_vecs * (int)sizeof(real4);
-   int cap = (share - kClearList * (int)sizeof(real_t *)) / (kSlotBytes + (int)sizeof(real_t *));
-   cap = cap > 64 ? 64 : (cap < 0 ? 0 : cap);
-   st.slots = lds + wave * p.stage_vecs;
-   st.to = reinterpret_cast<real_t **>(st.slots + cap * L * R);
-   st.clear = st.to + cap;
-   st.cap = cap;
+   int cap = (share - kClearList * (int)sizeof(real_t *)) /
+             (stage_width<V, L, R, EXACT, IdxT>(p) * (int)sizeof(real4) + (int)sizeof(real_t *));
+   cap = cap > 64 ? 64 : cap;
+   st.cap = (p.store_shift > 0 && cap >= 2 * S) ? cap : 0;     // room for two rows, or two packed groups, at least
    st.n = 0;
    st.nclear = 0;
-   st.shift = cap >= 2 * S ? p.store_shift : 0;     // room for two rows, or two packed groups, at least
-   st.tick = st.shift ? (unsigned int)(__builtin_amdgcn_s_memrealtime() >> st.shift) : 0u;
+   st.tick = st.cap ? (unsigned int)(__builtin_amdgcn_s_memrealtime() >> p.store_shift) : 0u;
 }
 
-template <int V, int L, int R, bool EXACT>
-__device__ __forceinline__ void stage_flush(RowStage &st, int lane, int k)
+template <int V, int L, int R, bool EXACT, typename IdxT>
+__device__ __forceinline__ void stage_flush(RowStage &st, const Params<IdxT> &p, int lane)
 {
    constexpr int S = 64 / L;
    const int sub = (L == 64) ? 0 : lane / L, sl = (L == 64) ? lane : lane % L;
+   const int width = stage_width<V, L, R, EXACT, IdxT>(p);
+   const real4 *slots = stage_slots<IdxT>(p);
+   real_t *const *to_list = stage_to<V, L, R, EXACT, IdxT>(p, st);
+   real_t *const *clear_list = to_list + st.cap;
    __builtin_amdgcn_wave_barrier();
    for (int i = 0; i < st.n; i += S)
    {
       const int slot = i + sub;
       if (slot < st.n)
       {
-         real_t *to = st.to[slot];
+         real_t *to = to_list[slot];
          if (to)
          {
             Slice<R> row;
 #pragma unroll
-            for (int r = 0; r < R; r++) row.v[r] = st.slots[(slot * R + r) * L + sl];
-            store_slice<V, L, R, EXACT, true>(to, row, sl, k);
+            for (int r = 0; r < R; r++)
+               row.v[r] = (V != 4 || EXACT || r * L + sl < width) ? slots[slot * width + r * L + sl] : zero4();
+            store_slice<V, L, R, EXACT, true>(to, row, sl, p.k);
          }
       }
    }
@@ -967,7 +997,7 @@ __device__ __forceinline__ void stage_flush(RowStage &st, int lane, int k)
          Slice<R> zero;
 #pragma unroll
          for (int r = 0; r < R; r++) zero.v[r] = zero4();
-         store_slice<V, L, R, EXACT, true>(st.clear[at], zero, sl, k);
+         store_slice<V, L, R, EXACT, true>(clear_list[at], zero, sl, p.k);
       }
    }
    __builtin_amdgcn_wave_barrier();
@@ -975,77 +1005,82 @@ __device__ __forceinline__ void stage_flush(RowStage &st, int lane, int k)
    st.nclear = 0;
 }
 
-// Has the tick passed?  Then everything waiting goes out.  `clock` is a reading of the 100 MHz counter taken a
-// little earlier (before the row was walked: the read is under way while the row is).
-template <int V, int L, int R, bool EXACT>
-__device__ __forceinline__ void stage_tick(RowStage &st, unsigned long long clock, int lane, int k)
+// Has the tick passed?  Then everything waiting goes out.  `clock` is a reading of the 100 MHz counter.
+template <int V, int L, int R, bool EXACT, typename IdxT>
+__device__ __forceinline__ void stage_tick(RowStage &st, const Params<IdxT> &p, unsigned long long clock, int lane)
 {
-   if (st.shift == 0) return;
-   const unsigned int now = (unsigned int)(clock >> st.shift);
+   if (st.cap == 0) return;
+   const unsigned int now = (unsigned int)(clock >> p.store_shift);
    if (now != st.tick)
    {
-      if (st.n | st.nclear) stage_flush<V, L, R, EXACT>(st, lane, k);
+      if (st.n | st.nclear) stage_flush<V, L, R, EXACT, IdxT>(st, p, lane);
       st.tick = now;
    }
 }
 
 // One finished row, held by the wavefront's first sub-wave; zrow is wave-uniform.
-template <int V, int L, int R, bool EXACT>
-__device__ __forceinline__ void stage_row(RowStage &st, real_t *zrow, const Slice<R> &acc, int lane, int k)
+template <int V, int L, int R, bool EXACT, typename IdxT>
+__device__ __forceinline__ void stage_row(RowStage &st, const Params<IdxT> &p, real_t *zrow, const Slice<R> &acc, int lane)
 {
    const int sub = (L == 64) ? 0 : lane / L, sl = (L == 64) ? lane : lane % L;
-   if (st.shift == 0)
+   if (st.cap == 0)
    {
-      if (sub == 0) store_slice<V, L, R, EXACT, true>(zrow, acc, sl, k);
+      if (sub == 0) store_slice<V, L, R, EXACT, true>(zrow, acc, sl, p.k);
       return;
    }
-   if (st.n >= st.cap) stage_flush<V, L, R, EXACT>(st, lane, k);   // (a packed group may have filled the last slot)
+   if (st.n >= st.cap) stage_flush<V, L, R, EXACT, IdxT>(st, p, lane);   // (a packed group may have filled the last slot)
+   const int width = stage_width<V, L, R, EXACT, IdxT>(p);
+   real4 *slots = stage_slots<IdxT>(p);
    if (sub == 0)
    {
 #pragma unroll
-      for (int r = 0; r < R; r++) st.slots[(st.n * R + r) * L + sl] = acc.v[r];
+      for (int r = 0; r < R; r++)
+         if (V != 4 || EXACT || r * L + sl < width) slots[st.n * width + r * L + sl] = acc.v[r];
    }
-   if (lane == 0) st.to[st.n] = zrow;
+   if (lane == 0) stage_to<V, L, R, EXACT, IdxT>(p, st)[st.n] = zrow;
    st.n++;
 }
 
 // One row per sub-wave (a packed group): sub-wave s holds a row for `zrow` (its own; nullptr: nothing to store).
-template <int V, int L, int R, bool EXACT>
-__device__ __forceinline__ void stage_group(RowStage &st, real_t *zrow, const Slice<R> &acc, int lane, int k)
+template <int V, int L, int R, bool EXACT, typename IdxT>
+__device__ __forceinline__ void stage_group(RowStage &st, const Params<IdxT> &p, real_t *zrow, const Slice<R> &acc, int lane)
 {
    constexpr int S = 64 / L;
    const int sub = lane / L, sl = lane % L;
-   if (st.shift == 0)
+   if (st.cap == 0)
    {
-      if (zrow) store_slice<V, L, R, EXACT, true>(zrow, acc, sl, k);
+      if (zrow) store_slice<V, L, R, EXACT, true>(zrow, acc, sl, p.k);
       return;
    }
-   if (st.n + S > st.cap) stage_flush<V, L, R, EXACT>(st, lane, k);
+   if (st.n + S > st.cap) stage_flush<V, L, R, EXACT, IdxT>(st, p, lane);
+   const int width = stage_width<V, L, R, EXACT, IdxT>(p);
+   real4 *slots = stage_slots<IdxT>(p);
    const int slot = st.n + sub;
 #pragma unroll
-   for (int r = 0; r < R; r++) st.slots[(slot * R + r) * L + sl] = acc.v[r];
-   if (sl == 0) st.to[slot] = zrow;
+   for (int r = 0; r < R; r++)
+      if (V != 4 || EXACT || r * L + sl < width) slots[slot * width + r * L + sl] = acc.v[r];
+   if (sl == 0) stage_to<V, L, R, EXACT, IdxT>(p, st)[slot] = zrow;
    st.n += S;
 }
 
 // An empty row under the overwrite rule: to be cleared; zrow is wave-uniform.
-template <int V, int L, int R, bool EXACT>
-__device__ __forceinline__ void stage_clear(RowStage &st, real_t *zrow, int lane, int k)
+template <int V, int L, int R, bool EXACT, typename IdxT>
+__device__ __forceinline__ void stage_clear(RowStage &st, const Params<IdxT> &p, real_t *zrow, int lane)
 {
    const int sub = (L == 64) ? 0 : lane / L, sl = (L == 64) ? lane : lane % L;
-   if (st.shift == 0)
+   if (st.cap == 0)
    {
       if (sub == 0)
       {
          Slice<R> zero;
 #pragma unroll
          for (int r = 0; r < R; r++) zero.v[r] = zero4();
-         store_slice<V, L, R, EXACT, true>(zrow, zero, sl, k);
+         store_slice<V, L, R, EXACT, true>(zrow, zero, sl, p.k);
       }
       return;
    }
-   if (st.nclear >= kClearList) stage_flush<V, L, R, EXACT>(st, lane, k);
-   if (lane == 0) st.clear[st.nclear] = zrow;
+   if (st.nclear >= kClearList) stage_flush<V, L, R, EXACT, IdxT>(st, p, lane);
+   if (lane == 0) (stage_to<V, L, R, EXACT, IdxT>(p, st) + st.cap)[st.nclear] = zrow;
    st.nclear++;
 }
 
@@ -1195,7 +1230,7 @@ __device__ __forceinline__ void packed_group(const Params<IdxT> &p, int64_t row_
       }
    }
    else stores = !generic && p.beta_zero && row < p.m;    // empty row under the overwrite rule: zeros
-   stage_group<V, L, R, EXACT>(st, stores ? zrow : nullptr, acc, lane, p.k);
+   stage_group<V, L, R, EXACT, IdxT>(st, p, stores ? zrow : nullptr, acc, lane);
 }
 
 // Does the row phase take the stretches of 64 chunks in scattered order?  When rows are claimed dynamically,
@@ -1532,10 +1567,12 @@ __device__ __forceinline__ void segments_phase(const Params<IdxT> &p, lds_table_
 
 // ---- phase B of the fused kernel: one wavefront per row ---------------------------
 template <int V, int L, int R, bool EXACT, int OP, int SOPK, int U, typename IdxT>
-__device__ __forceinline__ void rows_phase(const Params<IdxT> &p, lds_table_t tab, real4 *stage_lds)
+__device__ __forceinline__ void rows_phase(const Params<IdxT> &p, lds_table_t tab)
 {
+   // (the general pipeline's instances write rows as they finish: their large bodies lost 10 % to the added state and
+   // code -- general sigmoid K=128: 1.52 -> 1.68 ms -- and they are not the instances anyone runs at scale)
    RowStage st;
-   stage_begin<L, R, IdxT>(st, p, stage_lds);
+   stage_begin<V, L, R, EXACT, OP != OP_GENERIC, IdxT>(st, p);
    const int lane = threadIdx.x & 63;
    const int sub = lane / L, sl = lane % L;
    const bool reads_x = op_reads_x<OP>(p.imessage);
@@ -1608,9 +1645,8 @@ __device__ __forceinline__ void rows_phase(const Params<IdxT> &p, lds_table_t ta
             {
                // sub-wave s takes row row0 + g0 + s: its pointers are in lane g0 + s
                const IdxT gb = chunk_entry<L>(my_b, g0 + lane / L), ge = chunk_entry<L>(my_e, g0 + lane / L);
-               const unsigned long long clock = __builtin_amdgcn_s_memrealtime();
                packed_group<V, L, R, EXACT, OP, SOPK, U, IdxT>(p, row0 + g0, gb, ge > gb ? ge : gb, (int)md, lane, tab, st);
-               stage_tick<V, L, R, EXACT>(st, clock, lane, p.k);
+               stage_tick<V, L, R, EXACT, IdxT>(st, p, __builtin_amdgcn_s_memrealtime(), lane);
                packed_rows |= gmask;
             }
          }
@@ -1641,7 +1677,7 @@ __device__ __forceinline__ void rows_phase(const Params<IdxT> &p, lds_table_t ta
       {
          // empty row (about half the rows of an R-MAT graph): nothing to gather; the
          // overwrite rule still clears Z, every other rule leaves it alone
-         if (!generic && p.beta_zero) stage_clear<V, L, R, EXACT>(st, zrow, lane, p.k);
+         if (!generic && p.beta_zero) stage_clear<V, L, R, EXACT, IdxT>(st, p, zrow, lane);
          continue;
       }
       if (generic && aop == kAopNoop) continue;   // general semantics with no accumulate stage: Z is left alone
@@ -1692,8 +1728,10 @@ __device__ __forceinline__ void rows_phase(const Params<IdxT> &p, lds_table_t ta
             for (int r = 0; r < R; r++) xs_next.v[r] = zero4();
          }
       }
-      const unsigned long long clock = __builtin_amdgcn_s_memrealtime();
       walk_edges<V, L, R, EXACT, OP, SOPK, U, IdxT>(acc, xs, p, jb, je, first, nb, ne, lane, tab);
+      // (the clock is read here, not before the walk, so that it is not one more value to keep through it; the read
+      // is under way while the sub-waves' sums are merged)
+      const unsigned long long clock = st.cap ? __builtin_amdgcn_s_memrealtime() : 0ull;
       merge_subwaves<L, R, OP>(acc, p.imessage);
 
       if (sub == 0 && !generic && !p.beta_zero)
@@ -1702,13 +1740,13 @@ __device__ __forceinline__ void rows_phase(const Params<IdxT> &p, lds_table_t ta
          load_slice<V, L, R, EXACT>(zin, zrow, sl, p.k);
          map2(acc, zin, acc, [](real_t a, real_t b) { return a + b; });
       }
-      stage_row<V, L, R, EXACT>(st, zrow, acc, lane, p.k);
-      stage_tick<V, L, R, EXACT>(st, clock, lane, p.k);
+      stage_row<V, L, R, EXACT, IdxT>(st, p, zrow, acc, lane);
+      stage_tick<V, L, R, EXACT, IdxT>(st, p, clock, lane);
    }
-   if (st.nclear) stage_tick<V, L, R, EXACT>(st, __builtin_amdgcn_s_memrealtime(), lane, p.k);   // a claim of empty rows
+   if (st.nclear) stage_tick<V, L, R, EXACT, IdxT>(st, p, __builtin_amdgcn_s_memrealtime(), lane);   // a claim of empty rows
    chunk = nc > 0 ? resolve_claim<IdxT>(p, claimed, cur, nc, nchunks, lane) : -1;
    }
-   if (st.n | st.nclear) stage_flush<V, L, R, EXACT>(st, lane, p.k);
+   if (st.n | st.nclear) stage_flush<V, L, R, EXACT, IdxT>(st, p, lane);
 }
 
 // Every wavefront ends here.  The last workgroup to finish, when nobody reads the
@@ -1765,15 +1803,14 @@ __device__ __forceinline__ void retire_wave(const Params<IdxT> &p)
 // rows (phase A), then claims ordinary rows until none are left (phase B).  One
 // kernel, so the short rows fill in behind the long segments instead of waiting
 // for them at a kernel boundary.
-extern __shared__ __attribute__((aligned(32))) unsigned char fmm_dynamic_lds[];
-
-template <int V, int L, int R, bool EXACT, int OP, int SOPK, int U, typename IdxT>
 // The float / int32 instances whose rows take one register per lane on sub-waves of 32 lanes or fewer are held to
-// 128 vector registers, four wavefronts per SIMD: they fit but for a few spilled values, and measured faster that
-// way than with the 130-145 registers the compiler takes when left alone (K=32 on 2^23 nodes: 3.18 against 3.42 ms;
-// K=64 on R-MAT 24: 23.1 against 23.7).  The wider instances and the other libraries keep the compiler's own
-// allocation: held to 128 registers, K=256 lost 2.5 %, and the int64 and double instances 4-6 % at K=64.
-#define FMM_MIN_WAVES ((R == 1 && L <= 32 && OP != OP_GENERIC && sizeof(IdxT) == 4 && sizeof(real_t) == 4) ? 4 : 1)
+// the residency they had before rows could wait in LDS -- 128 vector registers, four wavefronts per SIMD -- at the
+// price of a few spilled values (0-24 bytes per lane): measured faster that way than with the 130-145 registers the
+// compiler takes when left alone (K=32 on 2^23 nodes: 3.18 against 3.42 ms; K=64 on R-MAT 24: 23.1 against 23.7).
+// The wider instances, the general pipeline and the other libraries keep the compiler's own allocation: held to
+// 128 registers, K=256 lost 2.5 %, and the int64 and double instances 4-6 % at K=64.
+#define FMM_MIN_WAVES ((sizeof(IdxT) == 4 && sizeof(real_t) == 4 && R == 1 && L <= 32 && OP != OP_GENERIC) ? 4 : 1)
+template <int V, int L, int R, bool EXACT, int OP, int SOPK, int U, typename IdxT>
 __global__ __launch_bounds__(kBlockThreads, FMM_MIN_WAVES) void fused_kernel(const Params<IdxT> p)
 {
    __shared__ real_t lds_tab[(OP >= OP_DOT) ? kSigmoidTableSize : 1];
@@ -1781,7 +1818,7 @@ __global__ __launch_bounds__(kBlockThreads, FMM_MIN_WAVES) void fused_kernel(con
    const lds_table_t tab = stage_table(p.sigmoid_table, lds_tab, (OP >= OP_DOT) && uses_sop && (SOPK >= 0 ? SOPK : p.sop_kind) == SOP_SIGMOID);
    segments_phase<V, L, R, EXACT, OP, SOPK, U, IdxT>(p, tab);
    // finished Z rows wait in the dynamic LDS for the grid's common store tick
-   rows_phase<V, L, R, EXACT, OP, SOPK, U, IdxT>(p, tab, reinterpret_cast<real4 *>(fmm_dynamic_lds));
+   rows_phase<V, L, R, EXACT, OP, SOPK, U, IdxT>(p, tab);
    retire_wave<IdxT>(p);
 }
 

@@ -32,6 +32,7 @@ int launch_instance(const Params<idx_t> &p, const Launch &l)
       int lds = 163840 / want - (int)attr.sharedSizeBytes - 512;
       if (lds > 65536 - (int)attr.sharedSizeBytes) lds = 65536 - (int)attr.sharedSizeBytes;
       lds = lds > 0 ? lds / 1024 * 1024 : 0;
+      if (OP == OP_GENERIC) lds = 0;   // the general pipeline's instances write rows as they finish
       int got = occ;
       while (lds > 0)
       {

@@ -237,14 +237,15 @@ void fusedMM_amd_get_split(int64_t *heavy_deg, int *seg_len);
  * edges are summed (same values to rounding) and nothing else.  Returns the previous setting. */
 int fusedMM_amd_set_pack_rows(int enable);
 
-/* When finished rows of Z are written.  By default a finished row waits in the compute unit's local memory and
- * every wavefront of a call writes its waiting rows when the same tick of the device's constant 100 MHz counter
- * passes (the counter shifted right by `shift` bits: 13 is a period of 82 us), or earlier when its share of that
- * memory is full: the stores of the whole grid reach memory in short common bursts instead of a steady trickle
- * between the gathers, which the memory system serves faster.  Results do not change, bit for bit.  shift = 0
- * (FUSEDMM_STORE_TICK=off) writes every row as it finishes; 8 ... 24 sets the period; -1 (FUSEDMM_STORE_TICK=auto)
- * restores the default.  Rows too wide for two of them to fit the wavefront's share are always written at once.
- * Returns the previous setting.  For tests and experiments. */
+/* When finished rows of Z are written.  Where the gathered matrix Y is 1 GiB or more, a finished row waits in the
+ * compute unit's local memory and every wavefront of a call writes its waiting rows when the same tick of the
+ * device's constant 100 MHz counter passes (the counter shifted right by `shift` bits: 13, a period of 82 us; 12
+ * where the caller's nnz / m is below 10), or earlier when its share of that memory is full: the stores of the whole
+ * grid reach memory in short common bursts instead of a steady trickle between the gathers, which the memory system
+ * serves faster.  Results do not change, bit for bit.  shift = 0 (FUSEDMM_STORE_TICK=off) writes every row as it
+ * finishes; 8 ... 24 sets the period and holds rows whatever the size of Y; -1 (FUSEDMM_STORE_TICK=auto) restores
+ * the rule above.  Rows too wide for two of them to fit the wavefront's share, and the general pipeline's rows, are
+ * always written at once.  Returns the previous setting.  For tests and experiments. */
 int fusedMM_amd_set_store_tick(int shift);
 
 /*
