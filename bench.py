@@ -32,8 +32,9 @@ PEAK_HBM_GBPS = 8000.0
 TRAFFIC_IS = ("L2-miss (fabric) bytes per call: FETCH_SIZE + WRITE_SIZE scaled by a 1 GiB copy; served by HBM or by the "
               "256 MiB last-level cache, so an upper bound on HBM bytes")
 # Extra workloads of the default run, measured after the headline one and reported under "also":
-# the second configuration with a bandwidth target (gcn K=256), then the skewed ones.
-ALSO_DEFAULT = ("c3g", "c3", "c4", "c5")   # c3g and c3 share a graph
+# the second configuration with a bandwidth target (gcn K=256), then the skewed ones, then the middle of the reference's
+# own sweep of feature widths at HBM scale (K=128 on 2^23 nodes: nothing to reuse, nothing that fits a cache).
+ALSO_DEFAULT = ("c3g", "c3", "c4", "c5", "k128er")   # c3g and c3 share a graph
 PROFILE_OF = {"c2": "fused_kernel_sigmoid_k128_c2.md", "c3": "spmm_k256_c3_rmat22.md",
               "c3g": "gcn_k256_c3g_rmat22.md", "c4": "tdist_k64_c4_rmat24.md", "c5": "sigmoid_k512_c5_zipf.md",
               "k32er": "tdist_k32_k32er.md", "k64er": "tdist_k64_k64er.md", "k128er": "tdist_k128_k128er.md",

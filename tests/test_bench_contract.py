@@ -80,7 +80,7 @@ def test_the_default_run_also_times_the_other_bandwidth_target_and_the_skewed_gr
     with a bandwidth target) first, then the skewed graphs; each entry has its own roofline figures and spot check."""
     sys.path.insert(0, ROOT)
     import bench
-    assert bench.ALSO_DEFAULT[0] == "c3g" and set(bench.ALSO_DEFAULT) == {"c3g", "c4", "c5", "c3"}
+    assert bench.ALSO_DEFAULT[0] == "c3g" and set(bench.ALSO_DEFAULT) == {"c3g", "c4", "c5", "c3", "k128er"}
     assert all(w in bench.WORKLOADS and w in bench.PROFILE_OF for w in bench.ALSO_DEFAULT)
     full = {"value": 1.0, "unit": "GFLOP/s", "steps": 10, "warmup": 2, "ms_per_step": 2.0, "edges_per_s": 3.0,
             "config": {"workload": "c3g: x", "op": "g", "K": 256, "rows": 4, "nnz": 5, "graph_gen_s": 1.0, "store_tick": "auto",
