@@ -192,17 +192,21 @@ def test_random_structure_matches_the_mirror_bit_for_bit(seed):
     sk = SOP_NAMES[kind] if kind else 0
     split = gpu_api.default_split(k, vbits) if rng.random() < 0.4 else (int(rng.integers(20, 200)), int(rng.integers(8, 64)))
     pack = bool(rng.random() < 0.8)
+    # when finished rows are written: as they finish, on a 2.6 us or 82 us clock tick, or only when a wavefront's LDS is full
+    tick = int(rng.choice([0, 8, 13, 24]))
     print("case", seed, dict(bits=bits, vbits=vbits, rows=rows, cols=cols, k=k, op=tkern, beta=beta, ld=(ldx, ldy, ldz), m=m,
-                             split=split, pack=pack, nnz=nnz), flush=True)
+                             split=split, pack=pack, tick=tick, nnz=nnz), flush=True)
     lib = fa.load(bits, vbits)
     gpu_api.set_kind(sk, bits, vbits)
     gpu_api.set_split(split[0], split[1], bits, vbits)
     prev = lib.fusedMM_amd_set_pack_rows(1 if pack else 0)
+    prev_tick = lib.fusedMM_amd_set_store_tick(tick)
     try:
         rc, Z = gpu_api.run(MSG[tkern], g, X, Y, Z0, beta=beta, bits=bits, m=m, k=k, ldx=ldx, ldy=ldy, ldz=ldz, vbits=vbits)
     finally:
         gpu_api.set_split(0, 0, bits, vbits)
         lib.fusedMM_amd_set_pack_rows(prev)
+        lib.fusedMM_amd_set_store_tick(prev_tick)
     assert rc == 0
     want = gpu_api.oracle_mirror(orc(vbits), tkern, g, X, Y, Z0, beta, sk, k, split[0], split[1], m=m, pack=pack)
     np.testing.assert_array_equal(Z.view(u), want.view(u))

@@ -90,6 +90,57 @@ def test_general_pipeline_and_the_mirror():
         lib.fusedMM_amd_set_opt(prev_opt)
 
 
+@pytest.mark.parametrize("seed", range(8))
+def test_random_mixtures_of_row_lengths(seed):
+    """Tens of thousands of rows per call, so that every wavefront takes many of them: stretches of empty, short, medium
+    and long rows in random order (packed groups, whole-wavefront rows, rows to clear and rows cut into segments all
+    meet in one wavefront's share of LDS), random widths with and without idle lanes, strides wider than K, m < rows."""
+    from fusedmm_amd import synth
+    from test_gpu_random_cases import _random_degrees
+    rng = np.random.default_rng(4100 + seed)
+    rows, cols = int(rng.integers(60000, 150000)), int(rng.integers(2000, 50000))
+    k = [20, 32, 64, 100, 128, 160, 260, 512][seed]
+    tkern, kind = [("g", None), ("m", None), ("s", "sigmoid"), ("t", "tdist"), ("f", "fr")][seed % 5]
+    beta = float(seed % 2)
+    deg = _random_degrees(rng, rows)
+    deg[rng.integers(0, rows // 2, 3)] = [500, 2000, 7000]   # long rows among the first half (m covers them): cut into segments
+    rowptr = np.concatenate([[0], np.cumsum(deg)])
+    nnz = int(rowptr[-1])
+    g = synth.graph_from_rowptr(rows, cols, rowptr, rng.integers(0, cols, nnz, dtype=np.int64), None, 32)
+    g["val"] = synth.edge_values(nnz, seed)
+    ld = k + 4 * int(rng.integers(0, 3))
+    lo, hi = (-0.5, 0.5) if tkern in ("s", "g", "m") else (-1.0, 1.0)
+    X = graphs.features(rows, ld, seed, lo, hi, 1)
+    Y = graphs.features(cols, ld, seed, lo, hi, 2)
+    if tkern == "f":
+        Y = (Y + np.float32(3.0)).astype(np.float32)
+    Z0 = graphs.features(rows, ld, seed, -1, 1, 3)
+    m = rows if seed % 3 else int(rng.integers(rows // 2, rows))
+    sk = SOP_NAMES[kind] if kind else 0
+    lib = fa.load(32)
+    gpu_api.set_kind(sk, 32)
+    gpu_api.set_split(int(rng.integers(40, 400)), int(rng.integers(16, 128)), 32)
+    print("case", seed, dict(rows=rows, cols=cols, k=k, op=tkern, beta=beta, ld=ld, m=m, nnz=nnz), flush=True)
+    try:
+        out = {}
+        for shift in (0, 8, 24, 13):
+            prev = lib.fusedMM_amd_set_store_tick(shift)
+            try:
+                rc, Z = gpu_api.run(MSG[tkern], g, X, Y, Z0, beta=beta, m=m, k=k, ldx=ld, ldy=ld, ldz=ld)
+            finally:
+                lib.fusedMM_amd_set_store_tick(prev)
+            assert rc == 0
+            out[shift] = Z
+    finally:
+        gpu_api.set_split(0, 0, 32)
+    assert gpu_api.last_split()[1] > 0                      # some rows were cut into segments
+    for shift in (8, 24, 13):
+        np.testing.assert_array_equal(out[shift].view(np.uint32), out[0].view(np.uint32), err_msg="shift %d" % shift)
+    np.testing.assert_array_equal(out[0][m:], Z0[m:])
+    np.testing.assert_array_equal(out[0][:, k:], Z0[:, k:])
+    assert np.isfinite(out[0]).all()
+
+
 def test_setter_returns_the_previous_value_and_clamps():
     lib = fa.load(32)
     first = lib.fusedMM_amd_set_store_tick(12)
